@@ -208,6 +208,8 @@ class InferenceEngine:
         spec_k: int = 4,
         spec_ngram: int = 2,
         kv_dtype: str = "native",
+        kv_block_size: Optional[int] = None,
+        kv_blocks: Optional[int] = None,
     ) -> None:
         # cap on prompt tokens prefill-batched per step: bounds time-to-first
         # -token for requests behind a burst (they decode while later
@@ -263,16 +265,27 @@ class InferenceEngine:
         else:
             self.weights.random_init(seed=seed)
 
-        blocks_per_seq = -(-self.max_seq_len // kv_mod.BLOCK_SIZE)
-        n_blocks = max_batch * blocks_per_seq + kv_margin_blocks
+        block_size = kv_block_size or kv_mod.BLOCK_SIZE
+        blocks_per_seq = -(-self.max_seq_len // block_size)
+        # kv_blocks: an explicit pool size (pages shared by all live
+        # requests) instead of max_batch full-length sequences
+        n_blocks = (kv_blocks if kv_blocks is not None
+                    else max_batch * blocks_per_seq) + kv_margin_blocks
         # "fp8": OCP e4m3 KV pool — half the decode-attention bytes; the
         # chunked-prefill and speculative paths read the cache as bf16 and
         # are not fp8-enabled yet, so they are rejected up front
         self.kv_dtype = kv_dtype
         if kv_dtype == "fp8" and spec_decode:
             raise ValueError("fp8 KV does not support spec_decode yet")
+        hybrid = self.spec.is_hybrid
+        if hybrid and spec_decode:
+            # rejected proposals would have advanced the recurrent state
+            raise ValueError("speculative decoding is not available for "
+                             "stacks with recurrent state")
         self.kv = PagedKV(self.spec, self.device, dtype, n_blocks=n_blocks,
-                          kv_dtype=kv_dtype)
+                          block_size=block_size, kv_dtype=kv_dtype,
+                          # one slot per resident request + the scratch row
+                          n_state_slots=max_batch + 1 if hybrid else 0)
         self.runner = Runner(self.spec, self.weights, self.kv, self.device, dtype)
 
         # MoE captures while every decode bucket takes a capture-safe path:
@@ -286,6 +299,9 @@ class InferenceEngine:
             not self.spec.is_moe
             or Runner.moe_graph_capturable(self.spec, max_batch)
         )
+        if hybrid:
+            # the hybrid MoE captures only on its dense all-experts path
+            graphs_ok = on_gpu and max_batch <= Runner.MOE_DENSE_MAX_TOKENS
         self.use_graphs = graphs_ok if use_graphs is None else (use_graphs and graphs_ok)
         self.graphs: Optional[DecodeGraphs] = None
         if self.use_graphs:
@@ -598,41 +614,16 @@ class InferenceEngine:
         self._prefilling = list(queue_)
 
         dev = self.device
-        ids_list, pos_list, slot_list, cu = [], [], [], [0]
+        chunks = []
         for a, start, take in batch:
-            p = a.req.prompt_ids
-            self.kv.extend_seq(a.seq_id, start + take)
             a.prefilled = a.length = start + take
-            ids_list.extend(p[start : start + take])
-            pos_list.extend(range(start, start + take))
-            slot_list.extend(
-                self.kv.slot_mapping(a.seq_id, range(start, start + take))
-            )
-            cu.append(cu[-1] + take)
-        input_ids = torch.tensor(ids_list, dtype=torch.int64).to(dev, non_blocking=True)
-        positions = torch.tensor(pos_list, dtype=torch.int32).to(dev, non_blocking=True)
-        slots = torch.tensor(slot_list, dtype=torch.int32).to(dev, non_blocking=True)
-        cu_seqlens = torch.tensor(cu, dtype=torch.int32).to(dev, non_blocking=True)
-        max_len = max(take for _, _, take in batch)
+            chunks.append((a.seq_id, a.req.prompt_ids[start : start + take],
+                           start))
         whole = all(
             start == 0 and take == len(a.req.prompt_ids)
             for a, start, take in batch
         )
-        if whole:
-            hidden = self.runner.forward_prefill(
-                input_ids, positions, slots, cu_seqlens, max_len
-            )
-        else:
-            bt = self.kv.block_table([a.seq_id for a, _, _ in batch])
-            seq_lens = torch.tensor([start + take for _, start, take in batch],
-                dtype=torch.int32, device=dev,
-            )
-            query_lens = torch.tensor(
-                [take for _, _, take in batch], dtype=torch.int32).to(dev, non_blocking=True)
-            hidden = self.runner.forward_prefill(
-                input_ids, positions, slots, cu_seqlens, max_len,
-                block_table=bt, seq_lens=seq_lens, query_lens=query_lens,
-            )
+        hidden, cu = self._run_chunks(chunks, whole)
         self._prefilling = [
             a
             for a, start, take in batch
@@ -658,6 +649,98 @@ class InferenceEngine:
                 self._pen_release(a)
             else:
                 self._active.append(a)
+
+    @torch.no_grad()
+    def _run_chunks(self, chunks: List[tuple], whole: bool = False):
+        """One packed forward over [(seq_id, tokens, start)] chunks: grows
+        each sequence's pages to start+len(tokens), stores the chunk's cache
+        rows and attends to the paged history. `whole` (every chunk is a
+        complete prompt from position 0) lets dense stacks take the
+        cache-free varlen kernel. Returns (hidden [T, H], cu list)."""
+        dev = self.device
+        ids_list, pos_list, slot_list, cu = [], [], [], [0]
+        for seq_id, toks, start in chunks:
+            take = len(toks)
+            self.kv.extend_seq(seq_id, start + take)
+            ids_list.extend(toks)
+            pos_list.extend(range(start, start + take))
+            slot_list.extend(
+                self.kv.slot_mapping(seq_id, range(start, start + take))
+            )
+            cu.append(cu[-1] + take)
+        input_ids = torch.tensor(ids_list, dtype=torch.int64).to(dev, non_blocking=True)
+        positions = torch.tensor(pos_list, dtype=torch.int32).to(dev, non_blocking=True)
+        slots = torch.tensor(slot_list, dtype=torch.int32).to(dev, non_blocking=True)
+        cu_seqlens = torch.tensor(cu, dtype=torch.int32).to(dev, non_blocking=True)
+        max_len = max(len(toks) for _, toks, _ in chunks)
+        seqs = [seq_id for seq_id, _, _ in chunks]
+        if self.spec.is_hybrid:
+            hidden = self.runner.forward_prefill(
+                input_ids, positions, slots, cu_seqlens, max_len,
+                block_table=self.kv.block_table(seqs),
+                state_slots=self.kv.state_slots(seqs),
+            )
+        elif whole:
+            hidden = self.runner.forward_prefill(
+                input_ids, positions, slots, cu_seqlens, max_len
+            )
+        else:
+            bt = self.kv.block_table(seqs)
+            seq_lens = torch.tensor(
+                [start + len(toks) for _, toks, start in chunks],
+                dtype=torch.int32, device=dev,
+            )
+            query_lens = torch.tensor(
+                [len(toks) for _, toks, _ in chunks], dtype=torch.int32
+            ).to(dev, non_blocking=True)
+            hidden = self.runner.forward_prefill(
+                input_ids, positions, slots, cu_seqlens, max_len,
+                block_table=bt, seq_lens=seq_lens, query_lens=query_lens,
+            )
+        return hidden, cu
+
+    # ------------------------------------------------------- forced tokens
+
+    @torch.no_grad()
+    def feed(self, entries: List[tuple], end=()) -> Optional[torch.Tensor]:
+        """Forced-token step (trace replay, scoring): entries are
+        (request id, next tokens, wanted row indices among them). All
+        entries run as ONE packed batch through the same chunk forward the
+        scheduler's prefill uses, against the pages and state earlier calls
+        left; a request is admitted at its first entry and may sit out a
+        call. Requests named in `end` give their pages and state slot back
+        after the call. Returns fp32 logits [n_wanted, vocab] in entry
+        order (None if nothing is wanted). Not to be mixed with submit()
+        traffic on the same engine."""
+        fed = self.__dict__.setdefault("_fed", {})
+        chunks, rows, base = [], [], 0
+        for rid, toks, want in entries:
+            if not toks:
+                continue
+            a = fed.get(rid)
+            if a is None:
+                if len(fed) >= self.max_batch:
+                    raise RuntimeError("more live requests than max_batch")
+                seq_id = self._next_seq
+                self._next_seq += 1
+                self.kv.new_seq(seq_id)
+                a = fed[rid] = _Active(None, seq_id, 0)
+            chunks.append((a.seq_id, list(toks), a.length))
+            a.length += len(toks)
+            rows.extend(base + w for w in want)
+            base += len(toks)
+        logits = None
+        if chunks:
+            hidden, _ = self._run_chunks(chunks)
+            if rows:
+                idx = torch.tensor(rows, dtype=torch.int64).to(
+                    self.device, non_blocking=True)
+                logits = self.runner.lm_head(hidden[idx]).float()
+        for rid in end:
+            a = fed.pop(rid, None)
+            if a is not None:
+                self.kv.free_seq(a.seq_id)
+        return logits
 
     @torch.no_grad()
     def _decode_once(self) -> None:
@@ -737,12 +820,15 @@ class InferenceEngine:
                     "pos": torch.tensor([a.length for a in self._active], dtype=torch.int32).to(dev, non_blocking=True),
                     "lens": torch.tensor([a.length + 1 for a in self._active], dtype=torch.int32).to(dev, non_blocking=True),
                     "bt": self.kv.block_table(seqs),
+                    "state": (self.kv.state_slots(seqs)
+                              if self.spec.is_hybrid else None),
                 }
                 self._eager_state = st
                 self._dec_seqs = list(seqs)
             slots = decode_slot_mapping(st["bt"], st["pos"], self.kv.block_size)
             hidden = self.runner.forward_decode(
-                st["ids"], st["pos"], slots, st["bt"], st["lens"]
+                st["ids"], st["pos"], slots, st["bt"], st["lens"],
+                state_slots=st["state"],
             )
             logits = self.runner.lm_head(hidden)
 

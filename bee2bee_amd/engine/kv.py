@@ -6,6 +6,19 @@ blocks are handed to sequences from a free list. Layout
 [n_blocks, n_kv_heads, block_size, head_dim] keeps one (key, head) row
 contiguous (256 B for hd=128 bf16) — the decode kernel reads it as 64 lanes
 x 4 B, a perfectly coalesced wave read.
+
+Hybrid stacks (spec.layer_specs) get a different pool per layer kind from
+the SAME page and slot bookkeeping:
+  * latent-attention layers: one page pool [n_blocks, block_size,
+    kv_rank + rot_dim] — the normed latent and the shared rotated key part
+    of each token (k_cache[i]; there is no separate value pool);
+  * linear-attention layers: no pages, a recurrent state
+    [n_slots, heads, dim, vdim] fp32 per sequence slot;
+  * every layer with an input convolution: the last taps-1 mixer inputs
+    [n_slots, taps-1, width] per sequence slot.
+A sequence owns one state slot from new_seq to free_seq. Slots and pages
+are handed out again without clearing: the kernels never read state or
+cache rows that precede a sequence's position 0.
 """
 from __future__ import annotations
 
@@ -33,6 +46,7 @@ class PagedKV:
         block_size: int = BLOCK_SIZE,
         layer_range: Optional[Tuple[int, int]] = None,
         kv_dtype: str = "native",
+        n_state_slots: int = 0,
     ) -> None:
         """kv_dtype: "native" stores the compute dtype; "fp8" stores OCP
         e4m3 bytes (uint8 pool, HALF the KV bytes — the decode kernels read
@@ -46,18 +60,66 @@ class PagedKV:
         lo, hi = layer_range or (0, spec.n_layers)
         self.layer_lo = lo
         store_dtype = torch.uint8 if kv_dtype == "fp8" else dtype
-        shape = (n_blocks, spec.n_kv_heads, block_size, spec.head_dim)
-        self.k_cache = [
-            torch.zeros(shape, device=device, dtype=store_dtype)
-            for _ in range(lo, hi)
-        ]
-        self.v_cache = [
-            torch.zeros(shape, device=device, dtype=store_dtype)
-            for _ in range(lo, hi)
-        ]
+        self.n_state_slots = 0
+        self._free_slots: List[int] = []
+        self._seq_slot: Dict[int, int] = {}
+        if spec.is_hybrid:
+            if kv_dtype != "native" or layer_range is not None:
+                raise ValueError(
+                    "hybrid stacks use the native cache dtype, unsharded")
+            self._init_hybrid(n_state_slots)
+        else:
+            shape = (n_blocks, spec.n_kv_heads, block_size, spec.head_dim)
+            self.k_cache = [
+                torch.zeros(shape, device=device, dtype=store_dtype)
+                for _ in range(lo, hi)
+            ]
+            self.v_cache = [
+                torch.zeros(shape, device=device, dtype=store_dtype)
+                for _ in range(lo, hi)
+            ]
         self._free: List[int] = list(range(n_blocks - 1, -1, -1))
         self._seq_blocks: Dict[int, List[int]] = {}
         self._seq_len: Dict[int, int] = {}
+
+    def _init_hybrid(self, n_slots: int) -> None:
+        spec, dev = self.spec, self.device
+        if n_slots <= 0:
+            raise ValueError("hybrid stacks need n_state_slots > 0")
+        self.n_state_slots = n_slots
+        self._free_slots = list(range(n_slots - 1, -1, -1))
+        self.k_cache, self.v_cache = [], []
+        self.conv_state: List[Optional[torch.Tensor]] = []
+        self.rec_state: List[Optional[torch.Tensor]] = []
+        taps = spec.canon_taps
+        for l in spec.layer_specs:
+            m = l.mixer
+            latent = m.kind == "latent_attention"
+            self.k_cache.append(torch.zeros(
+                self.n_blocks, self.block_size, m.cache_dim, device=dev,
+                dtype=self.dtype) if latent else None)
+            self.v_cache.append(None)
+            self.rec_state.append(None if latent else torch.zeros(
+                n_slots, m.heads, m.dim, m.vdim, device=dev,
+                dtype=torch.float32))
+            self.conv_state.append(torch.zeros(
+                n_slots, taps - 1, spec.hidden_size, device=dev,
+                dtype=self.dtype) if taps > 1 else None)
+
+    # ------------------------------------------------------- state slots
+
+    @property
+    def free_state_slots(self) -> int:
+        return len(self._free_slots)
+
+    def state_slot(self, seq_id: int) -> int:
+        return self._seq_slot[seq_id]
+
+    def state_slots(self, seq_ids: Sequence[int]) -> torch.Tensor:
+        """[B] int32 device tensor of the sequences' state slots."""
+        return torch.tensor([self._seq_slot[s] for s in seq_ids],
+                            dtype=torch.int32).to(self.device,
+                                                  non_blocking=True)
 
     def layer(self, layer_idx: int) -> Tuple[torch.Tensor, torch.Tensor]:
         return self.k_cache[layer_idx - self.layer_lo], self.v_cache[layer_idx - self.layer_lo]
@@ -69,6 +131,11 @@ class PagedKV:
     def new_seq(self, seq_id: int) -> None:
         if seq_id in self._seq_blocks:
             self.free_seq(seq_id)
+        if self.n_state_slots:
+            if not self._free_slots:
+                raise RuntimeError(
+                    f"state slots exhausted ({self.n_state_slots})")
+            self._seq_slot[seq_id] = self._free_slots.pop()
         self._seq_blocks[seq_id] = []
         self._seq_len[seq_id] = 0
 
@@ -76,6 +143,9 @@ class PagedKV:
         blocks = self._seq_blocks.pop(seq_id, [])
         self._seq_len.pop(seq_id, None)
         self._free.extend(reversed(blocks))
+        slot = self._seq_slot.pop(seq_id, None)
+        if slot is not None:
+            self._free_slots.append(slot)
 
     def seq_len(self, seq_id: int) -> int:
         return self._seq_len.get(seq_id, 0)

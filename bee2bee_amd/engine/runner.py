@@ -47,6 +47,14 @@ class Runner:
         # all-reduce their partial outputs over RCCL
         self.tp_group = None
         self.decode_attn_fn = None  # CP hook (parallel/cp.py)
+        # hybrid stacks: rotation tables per (dims, base) of their latent-
+        # attention layers, and an optional per-layer probe
+        # layer_tap(layer_idx, residual_fp32) for bring-up/debugging
+        self._rope_by_cfg = {}
+        self.layer_tap = None
+        if spec.is_hybrid:
+            self.rope_cos = self.rope_sin = None
+            return
         cos, sin = ops.rope_tables(
             spec.max_seq_len, spec.head_dim, spec.rope_theta, device,
             scaling=spec.rope_scaling,
@@ -81,6 +89,12 @@ class Runner:
         return ops.fused_add_rmsnorm(x, resid, w, self.spec.rms_eps)
 
     def lm_head(self, hidden: torch.Tensor) -> torch.Tensor:
+        if self.spec.is_hybrid:
+            # hidden is the fp32 residual stream; scalar-gain final norm
+            normed = ops.scalar_rmsnorm(
+                hidden.contiguous(), self.weights.final_gain,
+                self.spec.rms_eps, self.dtype)
+            return F.linear(normed, self.weights.lm_head)
         normed = self._norm(hidden, self.weights.final_norm,
                             self.weights.final_norm_bias)
         return F.linear(normed, self.weights.lm_head)
@@ -179,11 +193,25 @@ class Runner:
         return (cls.moe_grouped_aligned(spec)
                 and max_tokens <= cls.moe_grouped_max_tokens(spec))
 
-    def _moe_mlp(self, lw, x: torch.Tensor) -> torch.Tensor:
+    def _moe_mlp(self, lw, x: torch.Tensor, ffn=None) -> torch.Tensor:
         """Top-k expert MLP: dense all-experts bmm for decode-sized batches,
-        per-expert gather/GEMM/scatter for prefill-sized ones."""
+        per-expert gather/GEMM/scatter for prefill-sized ones.
+
+        ffn (models/hybrid.py MoEFFNSpec) overrides the uniform-stack
+        sizes per layer, routes on fp32 logits and swaps the activation for
+        the clamped GLU; routing (top-k, softmax over the chosen logits) and
+        the three execution strategies are shared."""
         s = self.spec
-        if self.ep is not None:
+        if ffn is not None:
+            E, I, top_k = ffn.n_experts, ffn.ff, ffn.top_k
+            logits = F.linear(x.float(), lw.moe_gate)
+
+            def act_fn(gu):
+                return ops.clamped_glu(gu, ffn.limit, ffn.alpha)
+        else:
+            E, I, top_k = s.n_experts, s.intermediate_size, s.top_k_experts
+            act_fn = ops.swiglu
+        if ffn is None and self.ep is not None:
             if self.weights.expert_range is not None:
                 # weights hold only this rank's expert shard (EP sharding)
                 w_gu, w_dn = lw.moe_w_gate_up, lw.moe_w_down
@@ -192,15 +220,15 @@ class Runner:
                 hi = lo + self.ep.local_e
                 w_gu, w_dn = lw.moe_w_gate_up[lo:hi], lw.moe_w_down[lo:hi]
             return self.ep.forward(x, lw.moe_gate, w_gu, w_dn)
-        logits = F.linear(x, lw.moe_gate)
-        weights, idx = ops.moe_topk_gate(logits, s.top_k_experts)  # [T,k]
+        if ffn is None:
+            logits = F.linear(x, lw.moe_gate)
+        weights, idx = ops.moe_topk_gate(logits, top_k)  # [T,k]
         T, H = x.shape
-        E, I = s.n_experts, s.intermediate_size
 
         if T <= self.MOE_DENSE_MAX_TOKENS:
             x_e = x.unsqueeze(0).expand(E, T, H)
             gu = torch.bmm(x_e, lw.moe_w_gate_up.transpose(1, 2))  # [E,T,2I]
-            act = ops.swiglu(gu.reshape(E * T, 2 * I)).view(E, T, I)
+            act = act_fn(gu.reshape(E * T, 2 * I)).view(E, T, I)
             y = torch.bmm(act, lw.moe_w_down.transpose(1, 2))  # [E,T,H]
             wfull = torch.zeros(T, E, dtype=torch.float32, device=x.device)
             wfull.scatter_(1, idx.long(), weights)
@@ -211,8 +239,9 @@ class Runner:
 
         use_grouped = (
             x.device.type == "cuda"
-            and self.moe_grouped_aligned(s)
-            and T <= self.moe_grouped_max_tokens(s)
+            and x.dtype == torch.bfloat16  # the kernel's only instantiation
+            and H % 128 == 0 and I % 128 == 0
+            and T <= self.MOE_GROUPED_ROWS * E // top_k
             and _os.environ.get("BEE2BEE_MOE_BMM") != "1"
         )
         # the padded bmm stays CPU-only (and opt-in for A/B measurement):
@@ -226,7 +255,7 @@ class Runner:
             # counting sort from one-hot cumsums: every op here (one_hot,
             # cumsum, gather, index_copy) is hipGraph-capture-safe —
             # torch.bincount/argsort are not
-            k = s.top_k_experts
+            k = top_k
             S = T * k
             flat_e = idx.reshape(-1).to(torch.int64)  # slot s -> expert
             oh = F.one_hot(flat_e, E)  # [S, E]
@@ -244,7 +273,7 @@ class Runner:
                 x_sorted = torch.empty(S, H, dtype=x.dtype, device=x.device)
                 x_sorted.index_copy_(0, pos, x[tok])
                 gu = ops.grouped_gemm(x_sorted, lw.moe_w_gate_up, offsets)
-                act = ops.swiglu(gu)
+                act = act_fn(gu)
                 y = ops.grouped_gemm(act, lw.moe_w_down, offsets)  # [S, H]
                 contrib = y[pos].float()  # back to slot order
             else:
@@ -258,7 +287,7 @@ class Runner:
                 padded = torch.zeros(E, C, H, dtype=x.dtype, device=x.device)
                 padded[flat_e, rank] = x[tok]
                 gu = torch.bmm(padded, lw.moe_w_gate_up.transpose(1, 2))
-                act = ops.swiglu(gu.reshape(E * C, 2 * I)).view(E, C, I)
+                act = act_fn(gu.reshape(E * C, 2 * I)).view(E, C, I)
                 y = torch.bmm(act, lw.moe_w_down.transpose(1, 2))  # [E,C,H]
                 contrib = y[flat_e, rank].float()  # [S, H] slot order
             out = torch.zeros(T, H, dtype=torch.float32, device=x.device)
@@ -275,7 +304,7 @@ class Runner:
             tok, kslot = mask.nonzero(as_tuple=True)
             xe = x[tok]
             ge = F.linear(xe, lw.moe_w_gate_up[e])
-            ye = F.linear(ops.swiglu(ge), lw.moe_w_down[e])
+            ye = F.linear(act_fn(ge), lw.moe_w_down[e])
             out.index_add_(0, tok, ye.float() * weights[tok, kslot, None])
         return out.to(x.dtype)
 
@@ -303,10 +332,17 @@ class Runner:
         block_table: Optional[torch.Tensor] = None,
         seq_lens: Optional[torch.Tensor] = None,
         query_lens: Optional[torch.Tensor] = None,
+        state_slots: Optional[torch.Tensor] = None,
     ) -> torch.Tensor:
         """Full- or chunked-prompt forward. Returns final hidden [T, H]
         (call lm_head on the rows you need). When seq_lens/query_lens are
         given the chunk attends to the paged history (chunked prefill)."""
+        if self.spec.is_hybrid:
+            # hybrid stacks always attend through the pages and carry
+            # per-sequence state; returns the fp32 residual stream
+            return self._forward_hybrid(
+                input_ids_or_hidden, positions, slot_mapping, cu_seqlens,
+                max_seqlen, block_table, state_slots)
         chunked = seq_lens is not None
 
         def attn(layer_idx, q, k, v, k_cache, v_cache):
@@ -335,9 +371,16 @@ class Runner:
         slot_mapping: torch.Tensor,
         block_table: torch.Tensor,
         seq_lens: torch.Tensor,
+        state_slots: Optional[torch.Tensor] = None,
     ) -> torch.Tensor:
         """One-token-per-sequence step. input [B] ids (or [B, H] hidden for
         later pipeline stages); returns final hidden [B, H]."""
+        if self.spec.is_hybrid:
+            B = input_ids_or_hidden.shape[0]
+            cu = torch.arange(B + 1, dtype=torch.int32, device=self.device)
+            return self._forward_hybrid(
+                input_ids_or_hidden, positions, slot_mapping, cu, 1,
+                block_table, state_slots)
 
         def attn(layer_idx, q, k, v, k_cache, v_cache):
             if self.decode_attn_fn is not None:
@@ -356,3 +399,115 @@ class Runner:
             else input_ids_or_hidden
         )
         return self._run_layers(hidden, positions, slot_mapping, attn)
+
+    # --------------------------------------------------------- hybrid stacks
+
+    def _rope_tables(self, dims: int, base: float):
+        key = (dims, base)
+        t = self._rope_by_cfg.get(key)
+        if t is None:
+            t = ops.rope_tables(self.spec.max_seq_len, dims, base, self.device)
+            self._rope_by_cfg[key] = t
+        return t
+
+    def _forward_hybrid(
+        self,
+        input_ids: torch.Tensor,
+        positions: torch.Tensor,
+        slot_mapping: torch.Tensor,
+        cu_seqlens: torch.Tensor,
+        max_qlen: int,
+        block_table: torch.Tensor,
+        state_slots: torch.Tensor,
+    ) -> torch.Tensor:
+        """One step of a hybrid stack over B packed chunks (prompt portions
+        and single decode tokens alike). The residual stream is fp32
+        end to end; each sublayer is normed before AND after:
+            x += g_post * unit(mixer(conv(g_pre * unit(x))))
+        and the post-norm + residual add + next pre-norm run as one fused
+        kernel. Returns the fp32 residual [T, width]."""
+        s, W = self.spec, self.weights
+        if block_table is None or state_slots is None:
+            raise ValueError("hybrid stacks need block_table and state_slots")
+        T = input_ids.shape[0]
+        B = cu_seqlens.shape[0] - 1
+        if max_qlen == 1:
+            seq_idx = cu_seqlens[:-1]
+        else:
+            lens = (cu_seqlens[1:] - cu_seqlens[:-1]).long()
+            seq_idx = torch.repeat_interleave(
+                torch.arange(B, dtype=torch.int32, device=self.device), lens,
+                output_size=T)
+        meta = (positions, slot_mapping, cu_seqlens, seq_idx, block_table,
+                state_slots, max_qlen)
+        x = F.embedding(input_ids, W.embed).float()
+        if s.embed_scale != 1.0:
+            x = x * s.embed_scale
+        normed = ops.scalar_rmsnorm(x, W.layers[0].gains[0], s.rms_eps,
+                                    self.dtype)
+        n = s.n_layers
+        for i in range(n):
+            nxt = W.layers[i + 1].gains[0] if i + 1 < n else None
+            normed = self._hybrid_layer(i, x, normed, meta, nxt)
+            if self.layer_tap is not None:
+                self.layer_tap(i, x)
+        return x
+
+    def _hybrid_layer(self, i: int, x: torch.Tensor, normed: torch.Tensor,
+                      meta, next_gain: Optional[float]):
+        """Updates the residual x in place; returns the next sublayer's
+        normed input (None after the last layer)."""
+        s = self.spec
+        lw, l = self.weights.layers[i], s.layer_specs[i]
+        (positions, slot_mapping, cu, seq_idx, block_table, state_slots,
+         max_qlen) = meta
+        m, eps, dt = l.mixer, s.rms_eps, self.dtype
+        T = normed.shape[0]
+        h = normed
+        if lw.canon is not None:
+            h = ops.canon_conv(h, lw.canon, self.kv.conv_state[i], state_slots,
+                               cu, seq_idx, positions)
+        proj = F.linear(h, lw.wqkv)
+        H = m.heads
+        if m.kind == "latent_attention":
+            D, R, C = m.dim, m.rot_dim, m.kv_rank
+            q = proj[:, : m.q_size].view(T, H, D + R)
+            kv = proj[:, m.q_size : m.q_size + m.cache_dim]
+            gate = proj[:, m.q_size + m.cache_dim :]
+            cache = self.kv.k_cache[i]
+            cos, sin = self._rope_tables(m.rope_dims, m.rope_base)
+            ops.latent_rope_store(q[..., D:], kv, lw.kv_norm, eps, C,
+                                  m.rope_dims, positions, cos, sin, cache,
+                                  slot_mapping)
+            # absorbed form: fold the key up-projection into the query and
+            # the value up-projection into the output, so attention runs on
+            # the cached latent rows directly (one shared row per token)
+            q_abs = torch.bmm(q[..., :D].transpose(0, 1), lw.w_uk)  # [H,T,C]
+            lat = ops.latent_attn(q_abs, q[..., D:], gate, cache, block_table,
+                                  positions, seq_idx, cu, m.window, m.scale,
+                                  max_qlen)
+            o = torch.bmm(lat, lw.w_uv)                          # [H,T,Dv]
+            y = F.linear(o.transpose(0, 1).reshape(T, H * m.vdim), lw.wo)
+        else:
+            HD, HV = H * m.dim, H * m.vdim
+            q = proj[:, :HD].view(T, H, m.dim)
+            k = proj[:, HD : 2 * HD].view(T, H, m.dim)
+            v = proj[:, 2 * HD : 2 * HD + HV].view(T, H, m.vdim)
+            gate = proj[:, 2 * HD + HV :]
+            o = ops.lightning_attn(q, k, v, lw.decay, self.kv.rec_state[i],
+                                   state_slots, cu, positions, max_qlen)
+            y = F.linear(ops.gated_rmsnorm(o, lw.out_norm, gate, eps, dt),
+                         lw.wo)
+        f = l.ffn
+        if f is None:
+            return ops.add_scalar_rmsnorm(x, y, lw.gains[1], next_gain, eps, dt)
+        normed2 = ops.add_scalar_rmsnorm(x, y, lw.gains[1], lw.gains[2], eps,
+                                         dt)
+        y = self._moe_mlp(lw, normed2, ffn=f)
+        y2 = None
+        if f.shared_ff:
+            gu = F.linear(normed2, lw.w_gate_up)
+            y2 = F.linear(ops.clamped_glu(gu, f.shared_limit, f.alpha),
+                          lw.w_down)
+        return ops.add_scalar_rmsnorm(x, y, lw.gains[3], next_gain, eps, dt,
+                                      y2=y2)

@@ -11,7 +11,7 @@ from __future__ import annotations
 import json
 import os
 from dataclasses import dataclass, field
-from typing import Any, Dict, Optional
+from typing import Any, Dict, List, Optional
 
 
 @dataclass
@@ -48,6 +48,16 @@ class ModelSpec:
     # vocab specials (byte-tokenizer defaults; overridden by a real tokenizer)
     bos_token_id: int = 1
     eos_token_id: int = 2
+    # hybrid stacks (arch "nukopel"): per-layer mixer/feed-forward specs
+    # (models/hybrid.py). When set, the uniform-layer fields above hold
+    # representative maxima only; the Runner's hybrid path reads these.
+    layer_specs: Optional[List[Any]] = None
+    embed_scale: float = 1.0     # x = embed[token] * embed_scale
+    canon_taps: int = 0          # causal per-channel conv on the mixer input
+
+    @property
+    def is_hybrid(self) -> bool:
+        return self.layer_specs is not None
 
     @property
     def is_moe(self) -> bool:
@@ -63,6 +73,11 @@ class ModelSpec:
 
     def n_params(self) -> int:
         """Parameter count (embeddings + layers + head)."""
+        if self.is_hybrid:
+            from .hybrid import hybrid_n_params
+
+            return hybrid_n_params(self.hidden_size, self.vocab_size,
+                                   self.canon_taps, self.layer_specs)
         h, i = self.hidden_size, self.intermediate_size
         attn = h * (self.q_size + 2 * self.kv_size) + self.q_size * h
         if self.is_moe:
@@ -79,6 +94,12 @@ class ModelSpec:
 
     def active_params_per_token(self) -> int:
         """Params touched per decoded token (MoE: only top-k experts)."""
+        if self.is_hybrid:
+            from .hybrid import hybrid_n_params
+
+            return hybrid_n_params(self.hidden_size, self.vocab_size,
+                                   self.canon_taps, self.layer_specs,
+                                   active_only=True)
         if not self.is_moe:
             return self.n_params()
         h, i = self.hidden_size, self.intermediate_size
@@ -392,6 +413,42 @@ _ALIASES = {
 }
 
 
+def hybrid_spec(name: str, vocab: int, width: int, layer_specs: List[Any],
+                *, eps: float, embed_scale: float, canon_taps: int,
+                max_seq_len: int = 32768) -> ModelSpec:
+    """ModelSpec for a hybrid stack (models/hybrid.py layer specs)."""
+    ffns = [l.ffn for l in layer_specs if l.ffn is not None]
+    return ModelSpec(
+        name=name, vocab_size=vocab, hidden_size=width,
+        intermediate_size=max([f.ff for f in ffns] or [0]),
+        n_layers=len(layer_specs),
+        n_heads=max(l.mixer.heads for l in layer_specs),
+        n_kv_heads=1,
+        head_dim=max(l.mixer.dim for l in layer_specs),
+        rms_eps=eps, max_seq_len=max_seq_len, tie_embeddings=False,
+        n_experts=max([f.n_experts for f in ffns] or [0]),
+        top_k_experts=max([f.top_k for f in ffns] or [0]),
+        arch="nukopel", norm_type="scalar_rmsnorm", act_type="clamped_glu",
+        pos_type="rope", layer_specs=list(layer_specs),
+        embed_scale=embed_scale, canon_taps=canon_taps,
+    )
+
+
+def nukopel_spec(name: str, cfg: Dict[str, Any]) -> ModelSpec:
+    """Parse a Nukopel config.json dict: every size and constant comes from
+    the file (layer order, per-layer mixer sizes, windows, decays, limits)."""
+    from .hybrid import layer_specs_from_cfg
+
+    return hybrid_spec(
+        name, int(cfg["vocab"]), int(cfg["width"]),
+        layer_specs_from_cfg(cfg["layers"]),
+        eps=float(cfg["norm"]["eps"]),
+        embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)),
+        canon_taps=int((cfg.get("canon") or {}).get("taps", 0)),
+        max_seq_len=int(cfg.get("max_seq_len", 32768)),
+    )
+
+
 def resolve_spec(name: str, model_path: Optional[str] = None) -> ModelSpec:
     """Resolve a model name (preset / alias / HF id / local dir) to a spec.
 
@@ -427,6 +484,9 @@ def spec_from_hf_config(model_path: str, name: Optional[str] = None) -> ModelSpe
     """Parse a HuggingFace config.json (Llama/Mistral/Mixtral/GPT-2 keys)."""
     with open(os.path.join(model_path, "config.json")) as f:
         cfg = json.load(f)
+    if cfg.get("architecture") == "Nukopel":
+        return nukopel_spec(
+            name or os.path.basename(os.path.normpath(model_path)), cfg)
     if cfg.get("model_type") == "gpt2" or "n_embd" in cfg:
         spec = _gpt2(
             name or cfg.get("_name_or_path", os.path.basename(model_path)),

@@ -35,6 +35,10 @@ class LayerWeights:
         "mlp_norm", "mlp_norm_bias",
         "w_gate_up", "w_gate_up_bias", "w_down", "w_down_bias",  # dense mlp
         "moe_gate", "moe_w_gate_up", "moe_w_down",  # moe
+        # hybrid stacks (models/hybrid.py): scalar norm gains, the input
+        # conv, the latent attention's norm / up-projections, the linear
+        # attention's output norm and per-head decay
+        "gains", "canon", "kv_norm", "w_uk", "w_uv", "out_norm", "decay",
     )
 
     def __init__(self) -> None:
@@ -53,6 +57,13 @@ class LayerWeights:
         self.moe_gate = None
         self.moe_w_gate_up = None
         self.moe_w_down = None
+        self.gains = None      # (pre-mixer, post-mixer, pre-ffn, post-ffn)
+        self.canon = None      # [width, taps] fp32
+        self.kv_norm = None    # [kv_rank] fp32
+        self.w_uk = None       # [heads, dim, kv_rank]
+        self.w_uv = None       # [heads, kv_rank, vdim]
+        self.out_norm = None   # [heads * vdim] fp32
+        self.decay = None      # [heads] fp32
 
 
 class ModelWeights:
@@ -65,6 +76,7 @@ class ModelWeights:
         self.final_norm: Optional[torch.Tensor] = None  # [hidden]
         self.final_norm_bias: Optional[torch.Tensor] = None
         self.lm_head: Optional[torch.Tensor] = None  # [vocab, hidden]
+        self.final_gain: Optional[float] = None  # scalar-gain final norm
         self.layers = [LayerWeights() for _ in range(spec.n_layers)]
         # expert-parallel shard: when set, MoE expert tensors hold only
         # experts [lo, hi) (gate stays replicated); see parallel/ep.py
@@ -88,6 +100,11 @@ class ModelWeights:
         shard — drawn per expert, so a shard holds exactly the values the
         full init would (EP-vs-single equivalence tests rely on this)."""
         s = self.spec
+        if s.is_hybrid:
+            if layer_range or expert_range:
+                raise NotImplementedError(
+                    "hybrid stacks are not sharded (pipeline/expert ranges)")
+            return self._random_init_hybrid(seed)
         lo, hi = layer_range or (0, s.n_layers)
         self.expert_range = expert_range
         e_lo, e_hi = expert_range or (0, getattr(s, "n_experts", 0) or 0)
@@ -180,6 +197,11 @@ class ModelWeights:
         """Load HF safetensors shards, fusing qkv / gate|up on the fly.
         expert_range: keep only that expert shard on device (EP ranks)."""
         s = self.spec
+        if s.is_hybrid:
+            if layer_range or expert_range:
+                raise NotImplementedError(
+                    "hybrid stacks are not sharded (pipeline/expert ranges)")
+            return self._load_nukopel(model_path)
         if s.arch == "gpt2":
             return self._load_gpt2(model_path, layer_range)
         lo, hi = layer_range or (0, s.n_layers)
@@ -373,6 +395,142 @@ class ModelWeights:
             self.lm_head = self.embed  # tied
         return self
 
+
+
+    # ------------------------------------------------------- hybrid stacks
+
+    @torch.no_grad()
+    def _load_nukopel(self, model_path: str) -> "ModelWeights":
+        """Nukopel safetensors: 'embed', 'head', 'final.norm', and per layer
+        'l<i>.norm1|norm1b|norm2|norm2b' (scalars), 'l<i>.canon1',
+        'l<i>.mix.*', 'l<i>.mlp.router|e<k>.*|shared.*'. All linear weights
+        are [out, in]."""
+        tensors = dict(iter_safetensors(model_path))
+        self._assemble_hybrid(lambda name: tensors.pop(name))
+        return self
+
+    @torch.no_grad()
+    def _random_init_hybrid(self, seed: int) -> "ModelWeights":
+        """Random weights under the checkpoint's tensor names, assembled by
+        the same code as a loaded checkpoint."""
+        import zlib
+
+        s = self.spec
+        W = s.hidden_size
+
+        def get(name: str) -> torch.Tensor:
+            tseed = (seed * 1000003 + zlib.crc32(name.encode())) % (2**31)
+            gen = torch.Generator(device=self.device).manual_seed(tseed)
+            shape, std = self._hybrid_shape(name)
+            t = torch.randn(*shape, generator=gen, dtype=torch.float32,
+                            device=self.device)
+            if std is None:               # gains / norm weights: around 1
+                return (1.0 + 0.1 * t).bfloat16()
+            return (t * std).bfloat16()
+
+        self._assemble_hybrid(get)
+        return self
+
+    def _hybrid_shape(self, name: str):
+        """(shape, init std or None for a gain) of a checkpoint tensor."""
+        s = self.spec
+        W, V = s.hidden_size, s.vocab_size
+        if name == "embed":
+            return (V, W), 1.0 / max(1.0, s.embed_scale)
+        if name == "head":
+            return (V, W), W ** -0.5
+        if name == "final.norm":
+            return (), None
+        parts = name.split(".")
+        l = s.layer_specs[int(parts[0][1:])]
+        m, f, rest = l.mixer, l.ffn, ".".join(parts[1:])
+        if rest in ("norm1", "norm1b", "norm2", "norm2b"):
+            return (), None
+        if rest == "canon1":
+            return (W, s.canon_taps), 0.2
+        if rest == "mix.o":
+            return (W, m.heads * m.vdim), (m.heads * m.vdim) ** -0.5
+        if rest == "mix.g":
+            rows = m.heads if m.kind == "latent_attention" else m.heads * m.vdim
+            return (rows, W), W ** -0.5
+        if m.kind == "latent_attention":
+            table = {"mix.q": ((m.q_size, W), W ** -0.5),
+                     "mix.dkv": ((m.cache_dim, W), W ** -0.5),
+                     "mix.dkv.norm": ((m.kv_rank,), None),
+                     "mix.uk": ((m.heads * m.dim, m.kv_rank), m.kv_rank ** -0.5),
+                     "mix.uv": ((m.heads * m.vdim, m.kv_rank), m.kv_rank ** -0.5)}
+        else:
+            table = {"mix.q": ((m.heads * m.dim, W), W ** -0.5),
+                     "mix.k": ((m.heads * m.dim, W), W ** -0.5),
+                     "mix.v": ((m.heads * m.vdim, W), W ** -0.5),
+                     "mix.norm": ((m.heads * m.vdim,), None)}
+        if rest in table:
+            return table[rest]
+        if rest == "mlp.router":
+            return (f.n_experts, W), W ** -0.5
+        ff = f.shared_ff if parts[2] == "shared" else f.ff
+        if parts[-1] == "down":
+            return (W, ff), ff ** -0.5
+        return (ff, W), W ** -0.5
+
+    def _assemble_hybrid(self, get) -> None:
+        """Build the engine layout from checkpoint-named tensors:
+        one fused input projection per mixer, per-head up-projection
+        stacks for the latent attention, stacked expert matrices."""
+        s = self.spec
+        dev, dt = self.device, self.dtype
+
+        def act(t: torch.Tensor) -> torch.Tensor:
+            return t.to(dev, dt).contiguous()
+
+        def f32(t: torch.Tensor) -> torch.Tensor:
+            return t.to(dev, torch.float32).contiguous()
+
+        def scalar(t: torch.Tensor) -> float:
+            return float(t.float().reshape(()))
+
+        self.embed = act(get("embed"))
+        self.lm_head = act(get("head"))
+        self.final_gain = scalar(get("final.norm"))
+        for i, l in enumerate(s.layer_specs):
+            lw, p, m, f = self.layers[i], f"l{i}.", l.mixer, l.ffn
+            lw.gains = tuple(
+                scalar(get(p + n))
+                if (f is not None or n in ("norm1", "norm1b")) else 1.0
+                for n in ("norm1", "norm1b", "norm2", "norm2b"))
+            if s.canon_taps:
+                lw.canon = f32(get(p + "canon1"))
+            if m.kind == "latent_attention":
+                # fused input projection rows: [q | latent+rot key | gate]
+                lw.wqkv = act(torch.cat([get(p + "mix.q"), get(p + "mix.dkv"),
+                                         get(p + "mix.g")], dim=0))
+                lw.kv_norm = f32(get(p + "mix.dkv.norm"))
+                lw.w_uk = act(get(p + "mix.uk").reshape(
+                    m.heads, m.dim, m.kv_rank))
+                lw.w_uv = act(get(p + "mix.uv").reshape(
+                    m.heads, m.vdim, m.kv_rank).transpose(1, 2))
+            else:
+                # fused input projection rows: [q | k | v | gate]
+                lw.wqkv = act(torch.cat([get(p + "mix.q"), get(p + "mix.k"),
+                                         get(p + "mix.v"), get(p + "mix.g")],
+                                        dim=0))
+                lw.out_norm = f32(get(p + "mix.norm"))
+                lw.decay = torch.tensor(m.decay, dtype=torch.float32,
+                                        device=dev)
+            lw.wo = act(get(p + "mix.o"))
+            if f is None:
+                continue
+            lw.moe_gate = f32(get(p + "mlp.router"))
+            lw.moe_w_gate_up = act(torch.stack([
+                torch.cat([get(f"{p}mlp.e{e}.gate"), get(f"{p}mlp.e{e}.up")],
+                          dim=0) for e in range(f.n_experts)]))
+            lw.moe_w_down = act(torch.stack([
+                get(f"{p}mlp.e{e}.down") for e in range(f.n_experts)]))
+            if f.shared_ff:
+                lw.w_gate_up = act(torch.cat(
+                    [get(p + "mlp.shared.gate"), get(p + "mlp.shared.up")],
+                    dim=0))
+                lw.w_down = act(get(p + "mlp.shared.down"))
 
 
 def _save_gpt2(weights: "ModelWeights", out_dir: str, tensors, cpu) -> None:

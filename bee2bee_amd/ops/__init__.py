@@ -235,3 +235,84 @@ def grouped_gemm(
     if _use_hip(x):
         return require_hip().grouped_gemm(x, w, offsets)
     return reference.grouped_gemm(x, w, offsets)
+
+
+# ------------------------------------------------------------ hybrid stacks
+# Mechanisms of the hybrid (latent-attention / linear-attention) layers.
+# Batch conventions: see ops/reference.py. Unlike the dense-transformer ops
+# above, these kernels are instantiated for bf16 AND fp32 activations; what
+# the designs compute in 32-bit (residual, norms, scores, recurrent state)
+# is fp32 in both.
+
+
+def scalar_rmsnorm(x, gain: float, eps: float, out_dtype):
+    if _use_hip(x):
+        return require_hip().scalar_rmsnorm(x, float(gain), eps, out_dtype)
+    return reference.scalar_rmsnorm(x, gain, eps, out_dtype)
+
+
+def add_scalar_rmsnorm(resid, y, post_gain: float, pre_gain, eps: float,
+                       out_dtype, y2=None):
+    """resid(fp32) += norm(y [+ y2])*post_gain in place; ->
+    norm(resid)*pre_gain (None when pre_gain is None). One fused pass on
+    GPU; y2 (e.g. a shared expert's output) is summed to y in fp32."""
+    if _use_hip(resid):
+        return require_hip().add_scalar_rmsnorm(
+            resid, y, y2, float(post_gain),
+            None if pre_gain is None else float(pre_gain), eps, out_dtype)
+    return reference.add_scalar_rmsnorm(resid, y, post_gain, pre_gain, eps,
+                                        out_dtype, y2=y2)
+
+
+def canon_conv(h, w, state, state_slots, cu_seqlens, seq_idx, positions):
+    if _use_hip(h):
+        return require_hip().canon_conv(h, w, state, state_slots, cu_seqlens,
+                                        seq_idx, positions)
+    return reference.canon_conv(h, w, state, state_slots, cu_seqlens, seq_idx,
+                                positions)
+
+
+def latent_rope_store(q_rot, kv, kv_norm, eps: float, kv_rank: int,
+                      rope_dims: int, positions, cos, sin, cache,
+                      slot_mapping) -> None:
+    if _use_hip(kv):
+        require_hip().latent_rope_store(q_rot, kv, kv_norm, eps, kv_rank,
+                                        rope_dims, positions, cos, sin, cache,
+                                        slot_mapping)
+        return
+    reference.latent_rope_store(q_rot, kv, kv_norm, eps, kv_rank, rope_dims,
+                                positions, cos, sin, cache, slot_mapping)
+
+
+def latent_attn(q_abs, q_rot, gate, cache, block_table, positions, seq_idx,
+                cu_seqlens, window: int, scale: float, max_qlen: int = 0):
+    """max_qlen: longest chunk in the batch (host int); 1 selects the
+    decode kernel, larger the query-tiled prefill kernel."""
+    if _use_hip(q_abs):
+        return require_hip().latent_attn(q_abs, q_rot, gate, cache,
+                                         block_table, positions, seq_idx,
+                                         window, scale, max_qlen)
+    return reference.latent_attn(q_abs, q_rot, gate, cache, block_table,
+                                 positions, seq_idx, cu_seqlens, window, scale)
+
+
+def lightning_attn(q, k, v, decay, state, state_slots, cu_seqlens, positions,
+                   max_qlen: int = 0):
+    if _use_hip(q):
+        return require_hip().lightning_attn(q, k, v, decay, state,
+                                            state_slots, cu_seqlens,
+                                            positions, max_qlen)
+    return reference.lightning_attn(q, k, v, decay, state, state_slots,
+                                    cu_seqlens, positions)
+
+
+def gated_rmsnorm(x, w, gate, eps: float, out_dtype):
+    if _use_hip(x):
+        return require_hip().gated_rmsnorm(x, w, gate, eps, out_dtype)
+    return reference.gated_rmsnorm(x, w, gate, eps, out_dtype)
+
+
+def clamped_glu(gate_up, limit: float, alpha: float):
+    if _use_hip(gate_up):
+        return require_hip().clamped_glu(gate_up, float(limit), float(alpha))
+    return reference.clamped_glu(gate_up, limit, alpha)

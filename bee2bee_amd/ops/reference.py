@@ -306,3 +306,215 @@ def attn_decode_lse(
     out = attn_decode(q, k_cache, v_cache, block_table, seq_lens, scale,
                       out_ml=out_ml)
     return out, out_ml
+
+
+# ------------------------------------------------------------ hybrid stacks
+#
+# Batch conventions for the varlen ops below (one step = B sequence chunks
+# packed into T rows; a decode token is a chunk of length 1):
+#   cu_seqlens  [B+1] int32   row range of each chunk
+#   seq_idx     [T]   int32   chunk index of each row
+#   positions   [T]   int32   absolute position of each row in its sequence
+#   state_slots [B]   int32   per-sequence state slot (conv / recurrent state)
+# State carried between steps is never trusted at a sequence's start: rows
+# whose source position is negative read zeros, and a chunk that starts at
+# position 0 starts from a zero recurrent state, so slots need no clearing.
+
+
+def scalar_rmsnorm(x: torch.Tensor, gain: float, eps: float,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """RMS norm with a single scalar gain: x / sqrt(mean(x^2) + eps) * g."""
+    xf = x.float()
+    r = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    return (xf * r * gain).to(out_dtype)
+
+
+def add_scalar_rmsnorm(resid: torch.Tensor, y: torch.Tensor, post_gain: float,
+                       pre_gain: Optional[float], eps: float,
+                       out_dtype: torch.dtype,
+                       y2: Optional[torch.Tensor] = None
+                       ) -> Optional[torch.Tensor]:
+    """resid (fp32, updated in place) += norm(y [+ y2]) * post_gain; returns
+    norm(resid) * pre_gain in out_dtype (None when pre_gain is None)."""
+    if y2 is not None:
+        y = y.float() + y2.float()
+    resid.add_(scalar_rmsnorm(y, post_gain, eps, torch.float32))
+    if pre_gain is None:
+        return None
+    return scalar_rmsnorm(resid, pre_gain, eps, out_dtype)
+
+
+def canon_conv(h: torch.Tensor, w: torch.Tensor, state: torch.Tensor,
+               state_slots: torch.Tensor, cu_seqlens: torch.Tensor,
+               seq_idx: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+    """h + causal per-channel conv over time. h [T, C]; w [C, taps] (tap
+    taps-1 multiplies the current row); state [n_slots, taps-1, C] holds each
+    sequence's last taps-1 inputs and is advanced in place."""
+    T, C = h.shape
+    K = w.shape[1] - 1
+    wf = w.float()
+    hf = h.float()
+    out = hf * (1.0 + wf[:, K])
+    if K == 0:
+        return out.to(h.dtype)
+    sidx = seq_idx.long()
+    rows = torch.arange(T, device=h.device)
+    local = rows - cu_seqlens.long()[sidx]
+    slots = state_slots.long()[sidx]
+    pos = positions.long()
+    for d in range(1, K + 1):
+        src_local = local - d
+        in_chunk = src_local >= 0
+        from_chunk = hf[(rows - d).clamp(min=0)]
+        from_state = state[slots, (K + src_local).clamp(0, K - 1)].float()
+        val = torch.where(in_chunk[:, None], from_chunk, from_state)
+        # select, never multiply: a reused slot may hold anything
+        val = torch.where((pos - d >= 0)[:, None], val, torch.zeros_like(val))
+        out += wf[:, K - d] * val
+    # advance the state: the last K inputs of each sequence after this chunk
+    cu = cu_seqlens.long()
+    B = cu.numel() - 1
+    lens = cu[1:] - cu[:-1]
+    kk = torch.arange(K, device=h.device)
+    src_local = lens[:, None] - K + kk[None, :]                  # [B, K]
+    in_chunk = src_local >= 0
+    from_chunk = h[(cu[:-1, None] + src_local).clamp(0, T - 1)]  # [B, K, C]
+    st = state_slots.long()
+    from_state = state[st[:, None], (K + src_local).clamp(0, K - 1)]
+    new = torch.where(in_chunk[..., None], from_chunk.to(state.dtype),
+                      from_state)
+    live = lens > 0
+    state[st[live]] = new[live]
+    return out.to(h.dtype)
+
+
+def _rot_half(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+              dims: int) -> torch.Tensor:
+    """Rotate the first `dims` coords of x [..., D] (pair i with i+dims/2);
+    cos/sin broadcast against x[..., :dims/2]."""
+    half = dims // 2
+    u, v = x[..., :half], x[..., half:dims]
+    return torch.cat([u * cos - v * sin, v * cos + u * sin, x[..., dims:]], -1)
+
+
+def latent_rope_store(q_rot: torch.Tensor, kv: torch.Tensor,
+                      kv_norm: torch.Tensor, eps: float, kv_rank: int,
+                      rope_dims: int, positions: torch.Tensor,
+                      cos: torch.Tensor, sin: torch.Tensor,
+                      cache: torch.Tensor, slot_mapping: torch.Tensor) -> None:
+    """q_rot [T, H, R] (view, rotated in place); kv [T, kv_rank + R] (view):
+    cache row = [rmsnorm(kv[:kv_rank]) * kv_norm | rotate(kv[kv_rank:])].
+    cache [n_blocks, block_size, kv_rank + R]."""
+    p = positions.long()
+    c, s = cos[p], sin[p]                                   # [T, dims/2]
+    q_rot.copy_(_rot_half(q_rot.float(), c[:, None], s[:, None],
+                          rope_dims).to(q_rot.dtype))
+    lat = kv[:, :kv_rank].float()
+    lat = lat * torch.rsqrt(lat.pow(2).mean(-1, keepdim=True) + eps) * kv_norm
+    kr = _rot_half(kv[:, kv_rank:].float(), c, s, rope_dims)
+    flat = cache.view(-1, cache.shape[-1])
+    flat[slot_mapping.long()] = torch.cat([lat, kr], -1).to(cache.dtype)
+
+
+def latent_attn(q_abs: torch.Tensor, q_rot: torch.Tensor, gate: torch.Tensor,
+                cache: torch.Tensor, block_table: torch.Tensor,
+                positions: torch.Tensor, seq_idx: torch.Tensor,
+                cu_seqlens: torch.Tensor, window: int,
+                scale: float) -> torch.Tensor:
+    """Windowed softmax attention in the latent space (one shared key/value
+    row per token). q_abs [H, T, C] (queries already multiplied by the key
+    up-projection), q_rot [T, H, R], gate [T, H] raw (sigmoid applied here).
+    Row t at position p of sequence b sees cached positions
+    max(0, p - window + 1) .. p. Returns [H, T, C] in q_abs.dtype."""
+    H, T, C = q_abs.shape
+    bs = cache.shape[1]
+    flat = cache.view(-1, cache.shape[-1])
+    out = torch.zeros(H, T, C, dtype=torch.float32, device=q_abs.device)
+    cu = cu_seqlens.tolist()
+    for b in range(len(cu) - 1):
+        lo, hi = cu[b], cu[b + 1]
+        if hi == lo:
+            continue
+        pos = positions[lo:hi].long()
+        k_lo = max(0, int(pos.min()) - window + 1)
+        k_hi = int(pos.max()) + 1
+        kpos = torch.arange(k_lo, k_hi, device=q_abs.device)
+        rows = block_table[b].long()[kpos // bs] * bs + kpos % bs
+        kv = flat[rows].float()                              # [S, C+R]
+        s = torch.einsum("htc,sc->hts", q_abs[:, lo:hi].float(), kv[:, :C])
+        s += torch.einsum("thr,sr->hts", q_rot[lo:hi].float(), kv[:, C:])
+        s *= scale
+        d = pos[:, None] - kpos[None, :]
+        s.masked_fill_(((d < 0) | (d >= window))[None], float("-inf"))
+        p = torch.softmax(s, dim=-1)
+        o = torch.einsum("hts,sc->htc", p, kv[:, :C])
+        out[:, lo:hi] = o * torch.sigmoid(gate[lo:hi].float()).t()[..., None]
+    return out.to(q_abs.dtype)
+
+
+LIGHTNING_CHUNK = 64
+
+
+def lightning_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                   decay: torch.Tensor, state: torch.Tensor,
+                   state_slots: torch.Tensor, cu_seqlens: torch.Tensor,
+                   positions: torch.Tensor) -> torch.Tensor:
+    """Decayed linear attention over packed chunks, fp32 throughout.
+    q,k [T, H, D], v [T, H, Dv] are RAW projections (silu applied here);
+    state [n_slots, H, D, Dv] fp32 is read (unless the chunk starts at
+    position 0) and advanced in place. Returns o [T, H * Dv] fp32 with
+    S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t."""
+    F = torch.nn.functional
+    T, H, D = q.shape
+    Dv = v.shape[-1]
+    out = torch.empty(T, H, Dv, dtype=torch.float32, device=q.device)
+    cu = cu_seqlens.tolist()
+    lam = decay.float()                                   # [H]
+    log_lam = torch.log(lam)
+    for b in range(len(cu) - 1):
+        lo, hi = cu[b], cu[b + 1]
+        if hi == lo:
+            continue
+        slot = int(state_slots[b])
+        if int(positions[lo]) == 0:
+            S = torch.zeros(H, D, Dv, dtype=torch.float32, device=q.device)
+        else:
+            S = state[slot].clone()
+        for c0 in range(lo, hi, LIGHTNING_CHUNK):
+            c1 = min(hi, c0 + LIGHTNING_CHUNK)
+            n = c1 - c0
+            qc = F.silu(q[c0:c1].float()).transpose(0, 1)   # [H, n, D]
+            kc = F.silu(k[c0:c1].float()).transpose(0, 1)
+            vc = F.silu(v[c0:c1].float()).transpose(0, 1)   # [H, n, Dv]
+            i = torch.arange(n, device=q.device, dtype=torch.float32)
+            diff = i[:, None] - i[None, :]                  # [n, n]
+            M = torch.exp(log_lam[:, None, None] * diff.clamp(min=0))
+            M = M * (diff >= 0)
+            a = torch.bmm(qc, kc.transpose(1, 2)) * M       # [H, n, n]
+            o = torch.bmm(a, vc)
+            carry = torch.exp(log_lam[:, None] * (i + 1.0))  # [H, n]
+            o += torch.bmm(qc, S) * carry[..., None]
+            out[c0:c1] = o.transpose(0, 1)
+            tail = torch.exp(log_lam[:, None] * (n - 1.0 - i))  # [H, n]
+            S = S * torch.exp(log_lam * n)[:, None, None] + torch.bmm(
+                (kc * tail[..., None]).transpose(1, 2), vc)
+        state[slot] = S
+    return out.view(T, H * Dv)
+
+
+def gated_rmsnorm(x: torch.Tensor, w: torch.Tensor, gate: torch.Tensor,
+                  eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """rmsnorm(x) * w * sigmoid(gate); x fp32 [T, N], gate raw [T, N]."""
+    xf = x.float()
+    r = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    return (xf * r * w.float() * torch.sigmoid(gate.float())).to(out_dtype)
+
+
+def clamped_glu(gate_up: torch.Tensor, limit: float,
+                alpha: float) -> torch.Tensor:
+    """[..., 2I] -> [..., I]: g = min(gate, limit), u = clamp(up, +-limit),
+    y = g * sigmoid(alpha * g) * (u + 1)."""
+    g, u = gate_up.float().chunk(2, dim=-1)
+    g = g.clamp(max=limit)
+    u = u.clamp(min=-limit, max=limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gate_up.dtype)
