@@ -1,0 +1,372 @@
+// Memory-bound kernels of the hybrid (latent-attention / linear-attention)
+// layer stacks: scalar-gain RMS norms fused with the fp32 residual update,
+// the causal per-channel input convolution with carried state, the latent
+// cache store (norm + rotation), the gated output norm and the clamped GLU.
+//
+// Every kernel is instantiated for bf16 (ushort bits) and fp32 activations;
+// the residual stream, norm statistics and rotation angles are fp32 in both.
+// Sequence starts are handled by position: rows whose source position is
+// negative read zeros (by select, never by multiply), so reused state slots
+// and cache pages need no clearing.
+#include "common.h"
+
+namespace {
+
+template <typename T> DEV_INLINE float ldf(const T* p);
+template <> DEV_INLINE float ldf<float>(const float* p) { return *p; }
+template <> DEV_INLINE float ldf<unsigned short>(const unsigned short* p) {
+    return bf2f(*p);
+}
+template <typename T> DEV_INLINE void stf(T* p, float v);
+template <> DEV_INLINE void stf<float>(float* p, float v) { *p = v; }
+template <> DEV_INLINE void stf<unsigned short>(unsigned short* p, float v) {
+    *p = f2bf(v);
+}
+
+// sum over the block (<= 1024 threads); every thread gets the total
+DEV_INLINE float block_sum(float v, float* red) {
+    v = wave_sum(v);
+    const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    __syncthreads();  // red may still be read from a previous reduction
+    if (lane == 0) red[wid] = v;
+    __syncthreads();
+    const int nw = (blockDim.x + WAVE - 1) / WAVE;
+    float total = 0.f;
+    for (int i = 0; i < nw; ++i) total += red[i];
+    return total;
+}
+
+// ------------------------------------------------------ scalar-gain norms
+// y = x / sqrt(mean(x^2) + eps) * gain; one workgroup per row, the row is
+// held in LDS between the passes.
+template <typename OT>
+__global__ void scalar_rmsnorm_kernel(const float* __restrict__ x,
+                                      OT* __restrict__ y, int W, float gain,
+                                      float eps) {
+    extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+    float* row = reinterpret_cast<float*>(smem_raw);
+    __shared__ float red[16];
+    const long t = blockIdx.x;
+    const float* xr = x + t * (long)W;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+        const float v = xr[i];
+        row[i] = v;
+        ss += v * v;
+    }
+    const float r = gain / sqrtf(block_sum(ss, red) / (float)W + eps);
+    OT* yr = y + t * (long)W;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) stf(yr + i, row[i] * r);
+}
+
+// resid += unit(y [+ y2]) * post_gain;  out = unit(resid) * pre_gain
+// (out skipped when HAS_OUT is false). One pass over HBM per operand.
+template <typename YT, typename OT, bool HAS_OUT>
+__global__ void add_scalar_rmsnorm_kernel(float* __restrict__ resid,
+                                          const YT* __restrict__ y,
+                                          const YT* __restrict__ y2,
+                                          OT* __restrict__ out, int W,
+                                          float post_gain, float pre_gain,
+                                          float eps) {
+    extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+    float* row = reinterpret_cast<float*>(smem_raw);
+    __shared__ float red[16];
+    const long t = blockIdx.x;
+    const YT* yr = y + t * (long)W;
+    const YT* y2r = y2 ? y2 + t * (long)W : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+        float v = ldf(yr + i);
+        if (y2r) v += ldf(y2r + i);
+        row[i] = v;
+        ss += v * v;
+    }
+    const float ry = post_gain / sqrtf(block_sum(ss, red) / (float)W + eps);
+    float* xr = resid + t * (long)W;
+    float sx = 0.f;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+        const float v = xr[i] + row[i] * ry;
+        xr[i] = v;
+        row[i] = v;
+        sx += v * v;
+    }
+    if (!HAS_OUT) return;
+    const float rx = pre_gain / sqrtf(block_sum(sx, red) / (float)W + eps);
+    OT* orow = out + t * (long)W;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) stf(orow + i, row[i] * rx);
+}
+
+// y = unit(x) * w * sigmoid(gate): x fp32 [T, N], gate raw with row stride
+template <typename T>
+__global__ void gated_rmsnorm_kernel(const float* __restrict__ x,
+                                     const float* __restrict__ w,
+                                     const T* __restrict__ gate,
+                                     long gate_stride, T* __restrict__ y,
+                                     int N, float eps) {
+    __shared__ float red[16];
+    const long t = blockIdx.x;
+    const float* xr = x + t * (long)N;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < N; i += blockDim.x) ss += xr[i] * xr[i];
+    const float r = 1.f / sqrtf(block_sum(ss, red) / (float)N + eps);
+    const T* gr = gate + t * gate_stride;
+    T* yr = y + t * (long)N;
+    for (int i = threadIdx.x; i < N; i += blockDim.x) {
+        const float g = 1.f / (1.f + expf(-ldf(gr + i)));
+        stf(yr + i, xr[i] * r * w[i] * g);
+    }
+}
+
+// ------------------------------------------------------------ clamped GLU
+// [rows, 2I] -> [rows, I]: g = min(gate, L), u = clamp(up, +-L),
+// y = g * sigmoid(alpha g) * (u + 1)
+template <typename T>
+__global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ y,
+                                   long rows, long I, float limit,
+                                   float alpha) {
+    const long n = rows * I;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < n;
+         idx += (long)gridDim.x * blockDim.x) {
+        const long r = idx / I, c = idx - r * I;
+        float g = ldf(gu + r * 2 * I + c);
+        float u = ldf(gu + r * 2 * I + I + c);
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        stf(y + idx, g / (1.f + expf(-alpha * g)) * (u + 1.f));
+    }
+}
+
+// ------------------------------------------------------- input convolution
+// out[t] = h[t] + sum_d w[c][K-d] * h[t-d], d = 0..K (K = taps-1). Rows
+// before the chunk come from the sequence's state (its last K inputs), rows
+// before position 0 are zero.
+template <typename T>
+__global__ void canon_conv_kernel(const T* __restrict__ h,
+                                  const float* __restrict__ w,   // [C, K+1]
+                                  const T* __restrict__ state,   // [S, K, C]
+                                  const int* __restrict__ state_slots,
+                                  const int* __restrict__ cu,
+                                  const int* __restrict__ seq_idx,
+                                  const int* __restrict__ positions,
+                                  T* __restrict__ out, int C, int K) {
+    const long t = blockIdx.x;
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const int b = seq_idx[t];
+    const int local = (int)t - cu[b];
+    const int pos = positions[t];
+    const long slot = state_slots[b];
+    const float* wc = w + (long)c * (K + 1);
+    float acc = ldf(h + t * C + c) * (1.f + wc[K]);
+    for (int d = 1; d <= K; ++d) {
+        if (pos - d < 0) break;
+        const int src = local - d;
+        const float v = src >= 0 ? ldf(h + (t - d) * C + c)
+                                 : ldf(state + (slot * K + (K + src)) * C + c);
+        acc += wc[K - d] * v;
+    }
+    stf(out + t * C + c, acc);
+}
+
+// state <- the sequence's last K inputs after this chunk (thread per
+// channel reads all K old rows before it writes any).
+template <typename T>
+__global__ void canon_state_kernel(const T* __restrict__ h,
+                                   T* __restrict__ state,
+                                   const int* __restrict__ state_slots,
+                                   const int* __restrict__ cu, int C, int K) {
+    const int b = blockIdx.x;
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const int lo = cu[b], L = cu[b + 1] - lo;
+    if (L <= 0) return;
+    T* st = state + (long)state_slots[b] * K * C + c;
+    T keep[8];
+    for (int k = 0; k < K; ++k) keep[k] = st[(long)k * C];
+    for (int k = 0; k < K; ++k) {
+        const int src = L - K + k;
+        st[(long)k * C] = src >= 0 ? h[(long)(lo + src) * C + c]
+                                   : keep[K + src];
+    }
+}
+
+// ----------------------------------------------------- latent cache store
+// Per token: cache row = [unit(kv[:C]) * w | rotate(kv[C:])]; q's rotated
+// parts are rotated in place. Rotation pairs dim i with i + dims/2 over the
+// first `dims` coords of the R-wide part; the rest pass through.
+template <typename T>
+__global__ void latent_rope_store_kernel(
+    T* __restrict__ q_rot, long q_tok_stride, long q_head_stride, int H,
+    const T* __restrict__ kv, long kv_stride, const float* __restrict__ w,
+    int C, int R, int dims, float eps, const int* __restrict__ positions,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    T* __restrict__ cache, const int* __restrict__ slot_mapping) {
+    __shared__ float red[16];
+    const long t = blockIdx.x;
+    const T* row = kv + t * kv_stride;
+    const long slot = slot_mapping[t];
+    T* dst = cache + slot * (long)(C + R);
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < C; i += blockDim.x) {
+        const float v = ldf(row + i);
+        ss += v * v;
+    }
+    const float r = 1.f / sqrtf(block_sum(ss, red) / (float)C + eps);
+    for (int i = threadIdx.x; i < C; i += blockDim.x)
+        stf(dst + i, ldf(row + i) * r * w[i]);
+    const int half = dims / 2;
+    const int p = positions[t];
+    const float* cs = cos_t + (long)p * half;
+    const float* sn = sin_t + (long)p * half;
+    for (int i = threadIdx.x; i < R; i += blockDim.x) {
+        float o;
+        if (i < half) {
+            o = ldf(row + C + i) * cs[i] - ldf(row + C + i + half) * sn[i];
+        } else if (i < dims) {
+            const int j = i - half;
+            o = ldf(row + C + i) * cs[j] + ldf(row + C + j) * sn[j];
+        } else {
+            o = ldf(row + C + i);
+        }
+        stf(dst + C + i, o);
+    }
+    // q: one thread per (head, pair) reads both coords, then writes both
+    T* qt = q_rot + t * q_tok_stride;
+    for (int i = threadIdx.x; i < H * half; i += blockDim.x) {
+        const int hh = i / half, j = i - hh * half;
+        T* qh = qt + hh * q_head_stride;
+        const float u = ldf(qh + j), v = ldf(qh + j + half);
+        stf(qh + j, u * cs[j] - v * sn[j]);
+        stf(qh + j + half, v * cs[j] + u * sn[j]);
+    }
+}
+
+}  // namespace
+
+// ------------------------------------------------------------- launchers
+// dtype codes: 0 = bf16 (ushort bits), 1 = fp32
+
+static inline int row_threads(int W) {
+    int th = 64;
+    while (th < W && th < 1024) th <<= 1;
+    return th > 256 && W < 2048 ? 256 : th;
+}
+
+extern "C" void launch_scalar_rmsnorm(const float* x, void* y, long T, int W,
+                                      float gain, float eps, int out_f32,
+                                      hipStream_t s) {
+    if (T == 0) return;
+    const int th = row_threads(W);
+    const size_t sh = (size_t)W * sizeof(float);
+    if (out_f32)
+        scalar_rmsnorm_kernel<float><<<T, th, sh, s>>>(x, (float*)y, W, gain, eps);
+    else
+        scalar_rmsnorm_kernel<unsigned short><<<T, th, sh, s>>>(
+            x, (unsigned short*)y, W, gain, eps);
+}
+
+template <typename YT, typename OT>
+static void add_norm_dispatch(float* resid, const void* y, const void* y2,
+                              void* out, long T, int W, float post, float pre,
+                              float eps, hipStream_t s) {
+    const int th = row_threads(W);
+    const size_t sh = (size_t)W * sizeof(float);
+    if (out)
+        add_scalar_rmsnorm_kernel<YT, OT, true><<<T, th, sh, s>>>(
+            resid, (const YT*)y, (const YT*)y2, (OT*)out, W, post, pre, eps);
+    else
+        add_scalar_rmsnorm_kernel<YT, OT, false><<<T, th, sh, s>>>(
+            resid, (const YT*)y, (const YT*)y2, (OT*)nullptr, W, post, pre, eps);
+}
+
+extern "C" void launch_add_scalar_rmsnorm(float* resid, const void* y,
+                                          const void* y2, void* out, long T,
+                                          int W, float post, float pre,
+                                          float eps, int y_f32, int out_f32,
+                                          hipStream_t s) {
+    if (T == 0) return;
+    if (y_f32 && out_f32)
+        add_norm_dispatch<float, float>(resid, y, y2, out, T, W, post, pre, eps, s);
+    else if (y_f32)
+        add_norm_dispatch<float, unsigned short>(resid, y, y2, out, T, W, post, pre, eps, s);
+    else if (out_f32)
+        add_norm_dispatch<unsigned short, float>(resid, y, y2, out, T, W, post, pre, eps, s);
+    else
+        add_norm_dispatch<unsigned short, unsigned short>(resid, y, y2, out, T, W, post, pre, eps, s);
+}
+
+extern "C" void launch_gated_rmsnorm(const float* x, const float* w,
+                                     const void* gate, long gate_stride,
+                                     void* y, long T, int N, float eps,
+                                     int f32, hipStream_t s) {
+    if (T == 0) return;
+    const int th = row_threads(N);
+    if (f32)
+        gated_rmsnorm_kernel<float><<<T, th, 0, s>>>(
+            x, w, (const float*)gate, gate_stride, (float*)y, N, eps);
+    else
+        gated_rmsnorm_kernel<unsigned short><<<T, th, 0, s>>>(
+            x, w, (const unsigned short*)gate, gate_stride,
+            (unsigned short*)y, N, eps);
+}
+
+extern "C" void launch_clamped_glu(const void* gu, void* y, long rows, long I,
+                                   float limit, float alpha, int f32,
+                                   hipStream_t s) {
+    const long n = rows * I;
+    if (n == 0) return;
+    const int th = 256;
+    long blocks = (n + th - 1) / th;
+    if (blocks > 65536) blocks = 65536;
+    if (f32)
+        clamped_glu_kernel<float><<<(int)blocks, th, 0, s>>>(
+            (const float*)gu, (float*)y, rows, I, limit, alpha);
+    else
+        clamped_glu_kernel<unsigned short><<<(int)blocks, th, 0, s>>>(
+            (const unsigned short*)gu, (unsigned short*)y, rows, I, limit, alpha);
+}
+
+extern "C" void launch_canon_conv(const void* h, const float* w, void* state,
+                                  const int* state_slots, const int* cu,
+                                  const int* seq_idx, const int* positions,
+                                  void* out, long T, int B, int C, int K,
+                                  int f32, hipStream_t s) {
+    if (T == 0) return;
+    const int th = C >= 256 ? 256 : 64;
+    const dim3 g1((unsigned)T, (C + th - 1) / th), g2(B, (C + th - 1) / th);
+    if (f32) {
+        canon_conv_kernel<float><<<g1, th, 0, s>>>(
+            (const float*)h, w, (const float*)state, state_slots, cu, seq_idx,
+            positions, (float*)out, C, K);
+        if (K > 0)
+            canon_state_kernel<float><<<g2, th, 0, s>>>(
+                (const float*)h, (float*)state, state_slots, cu, C, K);
+    } else {
+        canon_conv_kernel<unsigned short><<<g1, th, 0, s>>>(
+            (const unsigned short*)h, w, (const unsigned short*)state,
+            state_slots, cu, seq_idx, positions, (unsigned short*)out, C, K);
+        if (K > 0)
+            canon_state_kernel<unsigned short><<<g2, th, 0, s>>>(
+                (const unsigned short*)h, (unsigned short*)state, state_slots,
+                cu, C, K);
+    }
+}
+
+extern "C" void launch_latent_rope_store(
+    void* q_rot, long q_tok_stride, long q_head_stride, int H, const void* kv,
+    long kv_stride, const float* w, int C, int R, int dims, float eps,
+    const int* positions, const float* cos_t, const float* sin_t, void* cache,
+    const int* slot_mapping, long T, int f32, hipStream_t s) {
+    if (T == 0) return;
+    const int th = 256;
+    if (f32)
+        latent_rope_store_kernel<float><<<T, th, 0, s>>>(
+            (float*)q_rot, q_tok_stride, q_head_stride, H, (const float*)kv,
+            kv_stride, w, C, R, dims, eps, positions, cos_t, sin_t,
+            (float*)cache, slot_mapping);
+    else
+        latent_rope_store_kernel<unsigned short><<<T, th, 0, s>>>(
+            (unsigned short*)q_rot, q_tok_stride, q_head_stride, H,
+            (const unsigned short*)kv, kv_stride, w, C, R, dims, eps,
+            positions, cos_t, sin_t, (unsigned short*)cache, slot_mapping);
+}

@@ -1,0 +1,296 @@
+// Torch bindings for the hybrid-stack kernels (hybrid.hip, mixers.hip).
+// Shapes, strides and dtypes are validated here so the kernels index
+// without checks. Activations are bf16 or fp32 (the kernels are instantiated
+// for both); residual, norm weights and recurrent state are fp32. All entry
+// points are hipGraph-capture safe (no sync, no host reads).
+#include <torch/extension.h>
+#include <ATen/hip/HIPContext.h>
+#include <hip/hip_runtime.h>
+
+#include <optional>
+
+using torch::Tensor;
+
+extern "C" {
+void launch_scalar_rmsnorm(const float*, void*, long, int, float, float, int,
+                           hipStream_t);
+void launch_add_scalar_rmsnorm(float*, const void*, const void*, void*, long,
+                               int, float, float, float, int, int,
+                               hipStream_t);
+void launch_gated_rmsnorm(const float*, const float*, const void*, long,
+                          void*, long, int, float, int, hipStream_t);
+void launch_clamped_glu(const void*, void*, long, long, float, float, int,
+                        hipStream_t);
+void launch_canon_conv(const void*, const float*, void*, const int*,
+                       const int*, const int*, const int*, void*, long, int,
+                       int, int, int, hipStream_t);
+void launch_latent_rope_store(void*, long, long, int, const void*, long,
+                              const float*, int, int, int, float, const int*,
+                              const float*, const float*, void*, const int*,
+                              long, int, hipStream_t);
+int launch_latent_attn(const void*, const void*, long, long, const void*,
+                       long, const void*, const int*, int, const int*,
+                       const int*, void*, int, int, int, int, int, int, float,
+                       int, hipStream_t);
+int launch_lightning(const void*, const void*, const void*, long,
+                     const float*, float*, const int*, const int*, const int*,
+                     float*, int, int, int, int, int, hipStream_t);
+}
+
+namespace {
+
+inline hipStream_t stream() {
+    return at::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+}
+
+// 0 = bf16, 1 = fp32
+int act_code(at::ScalarType t, const char* name) {
+    TORCH_CHECK(t == torch::kBFloat16 || t == torch::kFloat32, name,
+                " must be bf16 or fp32");
+    return t == torch::kFloat32 ? 1 : 0;
+}
+
+int act_code(const Tensor& t, const char* name) {
+    TORCH_CHECK(t.is_cuda(), name, " must be on GPU");
+    return act_code(t.scalar_type(), name);
+}
+
+void check_f32(const Tensor& t, const char* name) {
+    TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kFloat32 &&
+                    t.is_contiguous(),
+                name, " must be a contiguous fp32 GPU tensor");
+}
+
+void check_i32(const Tensor& t, const char* name) {
+    TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kInt32 &&
+                    t.is_contiguous(),
+                name, " must be a contiguous int32 GPU tensor");
+}
+
+Tensor scalar_rmsnorm(const Tensor& x, double gain, double eps,
+                      at::ScalarType out_dtype) {
+    check_f32(x, "x");
+    TORCH_CHECK(x.dim() == 2);
+    const int oc = act_code(out_dtype, "out_dtype");
+    Tensor y = torch::empty(x.sizes(), x.options().dtype(out_dtype));
+    launch_scalar_rmsnorm(x.data_ptr<float>(), y.data_ptr(), x.size(0),
+                          (int)x.size(1), (float)gain, (float)eps, oc,
+                          stream());
+    return y;
+}
+
+std::optional<Tensor> add_scalar_rmsnorm(Tensor& resid, const Tensor& y,
+                                         const std::optional<Tensor>& y2,
+                                         double post_gain,
+                                         std::optional<double> pre_gain,
+                                         double eps,
+                                         at::ScalarType out_dtype) {
+    check_f32(resid, "resid");
+    TORCH_CHECK(resid.dim() == 2 && y.sizes() == resid.sizes() &&
+                y.is_contiguous());
+    const int yc = act_code(y, "y");
+    const int oc = act_code(out_dtype, "out_dtype");
+    const void* y2p = nullptr;
+    if (y2.has_value()) {
+        TORCH_CHECK(y2->sizes() == y.sizes() && y2->is_contiguous() &&
+                    y2->scalar_type() == y.scalar_type() && y2->is_cuda());
+        y2p = y2->data_ptr();
+    }
+    std::optional<Tensor> out;
+    void* op = nullptr;
+    if (pre_gain.has_value()) {
+        out = torch::empty(resid.sizes(), resid.options().dtype(out_dtype));
+        op = out->data_ptr();
+    }
+    launch_add_scalar_rmsnorm(resid.data_ptr<float>(), y.data_ptr(), y2p, op,
+                              resid.size(0), (int)resid.size(1),
+                              (float)post_gain,
+                              (float)pre_gain.value_or(1.0), (float)eps, yc,
+                              oc, stream());
+    return out;
+}
+
+Tensor gated_rmsnorm(const Tensor& x, const Tensor& w, const Tensor& gate,
+                     double eps, at::ScalarType out_dtype) {
+    check_f32(x, "x");
+    check_f32(w, "w");
+    TORCH_CHECK(x.dim() == 2 && w.numel() == x.size(1));
+    const int gc = act_code(gate, "gate");
+    TORCH_CHECK(gate.scalar_type() == out_dtype,
+                "gate and output share the activation dtype");
+    TORCH_CHECK(gate.dim() == 2 && gate.size(0) == x.size(0) &&
+                gate.size(1) == x.size(1) && gate.stride(1) == 1);
+    Tensor y = torch::empty(x.sizes(), x.options().dtype(out_dtype));
+    launch_gated_rmsnorm(x.data_ptr<float>(), w.data_ptr<float>(),
+                         gate.data_ptr(), gate.stride(0), y.data_ptr(),
+                         x.size(0), (int)x.size(1), (float)eps, gc, stream());
+    return y;
+}
+
+Tensor clamped_glu(const Tensor& gu, double limit, double alpha) {
+    const int c = act_code(gu, "gate_up");
+    TORCH_CHECK(gu.is_contiguous() && gu.size(-1) % 2 == 0);
+    const long I = gu.size(-1) / 2;
+    const long rows = gu.numel() / (2 * I);
+    auto shape = gu.sizes().vec();
+    shape.back() = I;
+    Tensor y = torch::empty(shape, gu.options());
+    launch_clamped_glu(gu.data_ptr(), y.data_ptr(), rows, I, (float)limit,
+                       (float)alpha, c, stream());
+    return y;
+}
+
+Tensor canon_conv(const Tensor& h, const Tensor& w, Tensor& state,
+                  const Tensor& state_slots, const Tensor& cu,
+                  const Tensor& seq_idx, const Tensor& positions) {
+    const int c = act_code(h, "h");
+    check_f32(w, "w");
+    check_i32(state_slots, "state_slots");
+    check_i32(cu, "cu_seqlens");
+    check_i32(seq_idx, "seq_idx");
+    check_i32(positions, "positions");
+    TORCH_CHECK(h.dim() == 2 && h.is_contiguous());
+    const long T = h.size(0);
+    const int C = (int)h.size(1), K = (int)w.size(1) - 1;
+    TORCH_CHECK(w.dim() == 2 && w.size(0) == C && K >= 0 && K <= 8,
+                "conv weight must be [channels, taps] with taps <= 9");
+    const int B = (int)cu.numel() - 1;
+    TORCH_CHECK(state_slots.numel() == B && seq_idx.numel() == T &&
+                positions.numel() == T);
+    if (K > 0)
+        TORCH_CHECK(state.is_cuda() && state.is_contiguous() &&
+                    state.scalar_type() == h.scalar_type() &&
+                    state.dim() == 3 && state.size(1) == K &&
+                    state.size(2) == C);
+    Tensor out = torch::empty_like(h);
+    launch_canon_conv(h.data_ptr(), w.data_ptr<float>(),
+                      K > 0 ? state.data_ptr() : nullptr,
+                      state_slots.data_ptr<int>(), cu.data_ptr<int>(),
+                      seq_idx.data_ptr<int>(), positions.data_ptr<int>(),
+                      out.data_ptr(), T, B, C, K, c, stream());
+    return out;
+}
+
+void latent_rope_store(Tensor& q_rot, const Tensor& kv, const Tensor& kv_norm,
+                       double eps, int64_t kv_rank, int64_t rope_dims,
+                       const Tensor& positions, const Tensor& cos_t,
+                       const Tensor& sin_t, Tensor& cache,
+                       const Tensor& slot_mapping) {
+    const int c = act_code(kv, "kv");
+    check_f32(kv_norm, "kv_norm");
+    check_f32(cos_t, "cos");
+    check_f32(sin_t, "sin");
+    check_i32(positions, "positions");
+    check_i32(slot_mapping, "slot_mapping");
+    TORCH_CHECK(q_rot.is_cuda() && q_rot.scalar_type() == kv.scalar_type() &&
+                cache.scalar_type() == kv.scalar_type() && cache.is_cuda());
+    TORCH_CHECK(q_rot.dim() == 3 && q_rot.stride(2) == 1);
+    TORCH_CHECK(kv.dim() == 2 && kv.stride(1) == 1);
+    const long T = kv.size(0);
+    const int R = (int)q_rot.size(2), C = (int)kv_rank;
+    TORCH_CHECK(kv.size(1) == C + R && q_rot.size(0) == T);
+    TORCH_CHECK(kv_norm.numel() == C);
+    TORCH_CHECK(rope_dims >= 0 && rope_dims <= R && rope_dims % 2 == 0);
+    TORCH_CHECK(cos_t.dim() == 2 && cos_t.size(1) == rope_dims / 2 &&
+                sin_t.sizes() == cos_t.sizes());
+    TORCH_CHECK(cache.is_contiguous() && cache.dim() == 3 &&
+                cache.size(2) == C + R);
+    TORCH_CHECK(positions.numel() == T && slot_mapping.numel() == T);
+    launch_latent_rope_store(
+        q_rot.data_ptr(), q_rot.stride(0), q_rot.stride(1),
+        (int)q_rot.size(1), kv.data_ptr(), kv.stride(0),
+        kv_norm.data_ptr<float>(), C, R, (int)rope_dims, (float)eps,
+        positions.data_ptr<int>(), cos_t.data_ptr<float>(),
+        sin_t.data_ptr<float>(), cache.data_ptr(),
+        slot_mapping.data_ptr<int>(), T, c, stream());
+}
+
+Tensor latent_attn(const Tensor& q_abs, const Tensor& q_rot,
+                   const Tensor& gate, const Tensor& cache,
+                   const Tensor& block_table, const Tensor& positions,
+                   const Tensor& seq_idx, int64_t window, double scale,
+                   int64_t max_qlen) {
+    const int c = act_code(q_abs, "q_abs");
+    check_i32(block_table, "block_table");
+    check_i32(positions, "positions");
+    check_i32(seq_idx, "seq_idx");
+    TORCH_CHECK(q_abs.dim() == 3 && q_abs.is_contiguous());
+    const int H = (int)q_abs.size(0), Tn = (int)q_abs.size(1),
+              C = (int)q_abs.size(2);
+    TORCH_CHECK(q_rot.is_cuda() && q_rot.scalar_type() == q_abs.scalar_type() &&
+                q_rot.dim() == 3 && q_rot.size(0) == Tn &&
+                q_rot.size(1) == H && q_rot.stride(2) == 1);
+    const int R = (int)q_rot.size(2);
+    TORCH_CHECK(gate.is_cuda() && gate.scalar_type() == q_abs.scalar_type() &&
+                gate.dim() == 2 && gate.size(0) == Tn && gate.size(1) == H &&
+                gate.stride(1) == 1);
+    TORCH_CHECK(cache.is_cuda() && cache.scalar_type() == q_abs.scalar_type() &&
+                cache.is_contiguous() && cache.dim() == 3 &&
+                cache.size(2) == C + R);
+    TORCH_CHECK(block_table.dim() == 2 && positions.numel() == Tn &&
+                seq_idx.numel() == Tn && window >= 1);
+    Tensor out = torch::empty_like(q_abs);
+    const int rc = launch_latent_attn(
+        q_abs.data_ptr(), q_rot.data_ptr(), q_rot.stride(0), q_rot.stride(1),
+        gate.data_ptr(), gate.stride(0), cache.data_ptr(),
+        block_table.data_ptr<int>(), (int)block_table.size(1),
+        positions.data_ptr<int>(), seq_idx.data_ptr<int>(), out.data_ptr(),
+        Tn, H, C, R, (int)cache.size(1), (int)window, (float)scale, c,
+        stream());
+    TORCH_CHECK(rc == 0, "latent_attn: kv_rank + rot_dim must be <= 1024");
+    return out;
+}
+
+Tensor lightning_attn(const Tensor& q, const Tensor& k, const Tensor& v,
+                      const Tensor& decay, Tensor& state,
+                      const Tensor& state_slots, const Tensor& cu,
+                      const Tensor& positions, int64_t max_qlen) {
+    const int c = act_code(q, "q");
+    check_f32(decay, "decay");
+    check_f32(state, "state");
+    check_i32(state_slots, "state_slots");
+    check_i32(cu, "cu_seqlens");
+    check_i32(positions, "positions");
+    TORCH_CHECK(q.dim() == 3 && k.sizes() == q.sizes() && v.dim() == 3);
+    const long T = q.size(0);
+    const int H = (int)q.size(1), D = (int)q.size(2), Dv = (int)v.size(2);
+    for (const Tensor* t : {&q, &k, &v}) {
+        TORCH_CHECK(t->is_cuda() && t->scalar_type() == q.scalar_type() &&
+                    t->size(0) == T && t->size(1) == H &&
+                    t->stride(2) == 1 &&
+                    (T == 1 || t->stride(0) == q.stride(0)) &&
+                    t->stride(1) == t->size(2));
+    }
+    TORCH_CHECK(decay.numel() == H);
+    TORCH_CHECK(state.dim() == 4 && state.size(1) == H &&
+                state.size(2) == D && state.size(3) == Dv);
+    const int B = (int)cu.numel() - 1;
+    TORCH_CHECK(state_slots.numel() == B && positions.numel() == T);
+    Tensor out = torch::empty({T, (long)H * Dv},
+                              q.options().dtype(torch::kFloat32));
+    const int rc = launch_lightning(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0),
+        decay.data_ptr<float>(), state.data_ptr<float>(),
+        state_slots.data_ptr<int>(), cu.data_ptr<int>(),
+        positions.data_ptr<int>(), out.data_ptr<float>(), B, H, D, Dv, c,
+        stream());
+    TORCH_CHECK(rc == 0, "lightning_attn: key dim must be <= 256");
+    return out;
+}
+
+}  // namespace
+
+void register_hybrid_ops(pybind11::module_& m) {
+    m.def("scalar_rmsnorm", &scalar_rmsnorm, "RMS norm with one scalar gain");
+    m.def("add_scalar_rmsnorm", &add_scalar_rmsnorm,
+          "resid += unit(y)*g_post; out = unit(resid)*g_pre");
+    m.def("gated_rmsnorm", &gated_rmsnorm, "unit(x) * w * sigmoid(gate)");
+    m.def("clamped_glu", &clamped_glu, "clamped GLU activation");
+    m.def("canon_conv", &canon_conv, "h + causal per-channel conv, carried state");
+    m.def("latent_rope_store", &latent_rope_store,
+          "latent norm + rotation + paged store; q rotation in place");
+    m.def("latent_attn", &latent_attn,
+          "windowed attention over the paged latent cache (absorbed form)");
+    m.def("lightning_attn", &lightning_attn,
+          "decayed linear attention with carried fp32 state");
+}

@@ -24,11 +24,17 @@ ext = CUDAExtension(
         os.path.join(CSRC, "attn_prefill.hip"),
         os.path.join(CSRC, "probe.hip"),
         os.path.join(CSRC, "grouped_gemm.hip"),
+        os.path.join(CSRC, "hybrid_ext.cpp"),
+        os.path.join(CSRC, "hybrid.hip"),
+        os.path.join(CSRC, "mixers.hip"),
     ],
     extra_compile_args={
         "cxx": ["-O3", "-std=c++17"]
         + (["-DBEE2BEE_DEBUG"] if os.environ.get("BEE2BEE_DEBUG_KERNELS") == "1" else []),
-        "nvcc": ["-O3", "-std=c++17", "--offload-arch=gfx950"]
+        # packed-fp32 VALU forms stay off: hipcc otherwise forms them from
+        # plain float code (the host pass warns it does not know the feature)
+        "nvcc": ["-O3", "-std=c++17", "--offload-arch=gfx950",
+                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
         + (["-DBEE2BEE_DEBUG", "-g"] if os.environ.get("BEE2BEE_DEBUG_KERNELS") == "1" else []),
     },
 )

@@ -1,0 +1,77 @@
+"""Nukopel served on the GPU (HIP kernels, bf16 and fp32) against the plain
+whole-sequence oracle: whole prompts, portions, decode, mixed batches with
+page/slot reuse, and greedy generation through the scheduler."""
+import pytest
+import torch
+
+from tests import nukopel_oracle as O
+from tests.nukopel_util import (chunk_schedule, make_engine, oracle_logits,
+                                random_tokens, rel_err, replay)
+
+pytestmark = pytest.mark.gpu
+
+if not torch.cuda.is_available():
+    pytest.skip("needs a GPU", allow_module_level=True)
+
+# bf16: rounding noise of a random-weight stack (the fp32 run is the sharp test)
+TOL = {torch.float32: 2e-4, torch.bfloat16: 0.15}
+
+
+def small_cfg():
+    return O.make_config(order=("lightning", "latent_attention", "lightning",
+                                "latent_attention"))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_whole_chunked_decode_match_oracle(tmp_path, dtype):
+    cfg = small_cfg()
+    W = O.random_weights(cfg, seed=1)
+    eng = make_engine(tmp_path, cfg, W, device="cuda", dtype=dtype)
+    toks = random_tokens(61, cfg["vocab"], 5)
+    want = oracle_logits(cfg, W, toks)
+    for sched in ([[("a", 61)]],
+                  chunk_schedule("a", 61, [2, 17, 3, 1, 1, 16]),
+                  [[("a", 20)]] + [[("a", 1)]] * 41):
+        got = replay(eng, {"a": toks}, sched)["a"]
+        assert rel_err(got, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_mixed_batches_reuse_pages_and_slots(tmp_path, dtype):
+    cfg = small_cfg()
+    W = O.random_weights(cfg, seed=2)
+    eng = make_engine(tmp_path, cfg, W, device="cuda", dtype=dtype,
+                      kv_blocks=12, block_size=16)
+    reqs = {f"r{i}": random_tokens(n, cfg["vocab"], 10 + i)
+            for i, n in enumerate([37, 9, 52, 18, 33, 5, 41])}
+    sched = [
+        [("r0", 20), ("r1", 2)],
+        [("r0", 1), ("r1", 7), ("r2", 30)],
+        [("r0", 16), ("r2", 1), ("r3", 18)],        # r0, r1, r3 end
+        [("r2", 21), ("r4", 33), ("r5", 2), ("r6", 3)],
+        [("r5", 3), ("r6", 38)],
+    ]
+    got = replay(eng, reqs, sched)
+    for rid, toks in reqs.items():
+        assert rel_err(got[rid], oracle_logits(cfg, W, toks)) < TOL[dtype], rid
+    assert eng.kv.free_state_slots == eng.kv.n_state_slots - 1
+
+
+def test_greedy_generation_through_scheduler(tmp_path):
+    cfg = small_cfg()
+    W = O.random_weights(cfg, seed=3)
+    eng = make_engine(tmp_path, cfg, W, device="cuda", dtype=torch.float32)
+    try:
+        prompt = random_tokens(11, cfg["vocab"], 3)
+        req = eng.generate(prompt, max_new_tokens=12, temperature=0.0,
+                           repetition_penalty=1.0)
+        seq = list(prompt)
+        for tok in req.output_ids:
+            logits = oracle_logits(cfg, W, seq)[-1]
+            top2 = torch.topk(logits, 2).values
+            if float(top2[0] - top2[1]) > 1e-3:   # skip near-ties
+                assert int(logits.argmax()) == tok
+            seq.append(tok)
+        assert len(req.output_ids) == 12
+    finally:
+        eng.shutdown()
