@@ -310,6 +310,10 @@ class InferenceEngine:
         self._scratch_seq = -1
         self.kv.new_seq(self._scratch_seq)
         self.kv.extend_seq(self._scratch_seq, 1)
+        if self.graphs is not None and hybrid:
+            self.graphs.scratch = (
+                self.kv.block_table([self._scratch_seq])[0],
+                self.kv.state_slot(self._scratch_seq))
 
         self._gen = torch.Generator(device=self.device)
         self._gen.manual_seed(seed)
@@ -794,12 +798,18 @@ class InferenceEngine:
                 )
                 bt = self.kv.block_table(seqs)
                 g.block_table[:B, : bt.shape[1]].copy_(bt, non_blocking=True)
+                if g.state_slots is not None:
+                    g.state_slots[:B].copy_(self.kv.state_slots(seqs),
+                                            non_blocking=True)
                 if bucket > B:  # pad rows -> scratch sequence, length 1
                     sb = self.kv.block_table([self._scratch_seq])[0]
                     g.block_table[B:bucket, : sb.shape[0]].copy_(sb)
                     g.positions[B:bucket].zero_()
                     g.seq_lens[B:bucket].fill_(1)
                     g.input_ids[B:bucket].zero_()
+                    if g.state_slots is not None:
+                        g.state_slots[B:bucket].fill_(
+                            self.kv.state_slot(self._scratch_seq))
                 self._dec_seqs = list(seqs)
             logits = g.run(B)[:B]
         else:
@@ -1298,6 +1308,9 @@ class InferenceEngine:
             g.positions[:batch].fill_(prompt_len)
             g.seq_lens[:batch].fill_(prompt_len + 1)
             g.block_table[:batch, : bt.shape[1]].copy_(bt)
+            if g.state_slots is not None:
+                g.state_slots[:batch].copy_(
+                    self.kv.state_slots([a.seq_id for a in acts]))
             bucket = g.bucket_for(batch)
             if bucket > batch:
                 sb = self.kv.block_table([self._scratch_seq])[0]
@@ -1305,6 +1318,9 @@ class InferenceEngine:
                 g.positions[batch:bucket].zero_()
                 g.seq_lens[batch:bucket].fill_(1)
                 g.input_ids[batch:bucket].zero_()
+                if g.state_slots is not None:
+                    g.state_slots[batch:bucket].fill_(
+                        self.kv.state_slot(self._scratch_seq))
             self._bench_state = ("graph", batch)
             self.graphs.run(batch)  # capture outside the timed region
             g.positions[:batch].fill_(prompt_len)
@@ -1316,6 +1332,8 @@ class InferenceEngine:
                 "pos": torch.full((batch,), prompt_len, dtype=torch.int32, device=dev),
                 "lens": torch.full((batch,), prompt_len + 1, dtype=torch.int32, device=dev),
                 "bt": bt,
+                "state": (self.kv.state_slots([a.seq_id for a in acts])
+                          if self.spec.is_hybrid else None),
             }
             self._bench_state = ("eager", batch)
 
@@ -1334,7 +1352,8 @@ class InferenceEngine:
             st = self._bench_eager
             slots = decode_slot_mapping(st["bt"], st["pos"], self.kv.block_size)
             hidden = self.runner.forward_decode(
-                st["ids"], st["pos"], slots, st["bt"], st["lens"]
+                st["ids"], st["pos"], slots, st["bt"], st["lens"],
+                state_slots=st["state"],
             )
             logits = self.runner.lm_head(hidden)
             st["ids"].copy_(torch.argmax(logits, dim=-1))

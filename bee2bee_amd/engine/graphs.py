@@ -45,6 +45,14 @@ class DecodeGraphs:
         self.block_table = torch.zeros(
             max_batch, self.width, dtype=torch.int32, device=dev
         )
+        # stacks with per-sequence recurrent/conv state: the state slot of
+        # each row, and the scratch row (block-table row, state slot) that
+        # capture-time warmup runs are pointed at — a warmup run ADVANCES
+        # state, so it must never touch a live sequence's slot
+        self.state_slots = (
+            torch.zeros(max_batch, dtype=torch.int32, device=dev)
+            if runner.spec.is_hybrid else None)
+        self.scratch = None  # (block_table row tensor, state slot int)
         self.logits: Dict[int, torch.Tensor] = {}
         self._graphs: Dict[int, torch.cuda.CUDAGraph] = {}
         self._pool = None
@@ -69,10 +77,35 @@ class DecodeGraphs:
         bt = self.block_table[:B]
         lens = self.seq_lens[:B]
         slots = decode_slot_mapping(bt, pos, self.runner.kv.block_size)
-        hidden = self.runner.forward_decode(ids, pos, slots, bt, lens)
+        st = None if self.state_slots is None else self.state_slots[:B]
+        hidden = self.runner.forward_decode(ids, pos, slots, bt, lens,
+                                            state_slots=st)
         return self.runner.lm_head(hidden)
 
     def _capture(self, B: int) -> None:
+        saved = None
+        if self.state_slots is not None:
+            # run warmup + capture against the scratch row, then put the
+            # caller's rows back
+            assert self.scratch is not None, "engine must set graphs.scratch"
+            bufs = (self.input_ids, self.positions, self.seq_lens,
+                    self.block_table, self.state_slots)
+            saved = [b[:B].clone() for b in bufs]
+            row, slot = self.scratch
+            self.input_ids[:B].zero_()
+            self.positions[:B].zero_()
+            self.seq_lens[:B].fill_(1)
+            self.block_table[:B, : row.shape[0]].copy_(row)
+            self.state_slots[:B].fill_(slot)
+        try:
+            self._capture_inner(B)
+        finally:
+            if saved is not None:
+                for b, sv in zip(bufs, saved):
+                    b[:B].copy_(sv)
+                torch.cuda.synchronize()
+
+    def _capture_inner(self, B: int) -> None:
         torch.cuda.synchronize()
         # warmup on a side stream (required before capture)
         s = torch.cuda.Stream()

@@ -104,7 +104,7 @@ class PagedKV:
                 dtype=torch.float32))
             self.conv_state.append(torch.zeros(
                 n_slots, taps - 1, spec.hidden_size, device=dev,
-                dtype=self.dtype) if taps > 1 else None)
+                dtype=self.dtype) if taps >= 1 else None)
 
     # ------------------------------------------------------- state slots
 

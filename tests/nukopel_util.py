@@ -29,12 +29,28 @@ def oracle_logits(cfg, W, tokens: Sequence[int]) -> torch.Tensor:
     return O.forward(list(tokens), W, cfg, dtype=torch.float64)[0]
 
 
-def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
-    """Row-wise RMS difference relative to the RMS of the expected logits
-    (max over rows)."""
+def row_errs(got: torch.Tensor, want: torch.Tensor) -> torch.Tensor:
+    """Per row: RMS difference relative to the RMS of the expected logits."""
     got, want = got.double().cpu(), want.double().cpu()
     d = (got - want).pow(2).mean(-1).sqrt()
-    return float((d / want.pow(2).mean(-1).sqrt().clamp_min(1e-12)).max())
+    return d / want.pow(2).mean(-1).sqrt().clamp_min(1e-12)
+
+
+def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    return float(row_errs(got, want).max())
+
+
+def assert_logits(got: torch.Tensor, want: torch.Tensor, dtype,
+                  what: str = "") -> None:
+    """fp32 runs must match the oracle row by row. bf16 runs carry rounding
+    noise, and a row whose router sees a near-tie may pick another expert:
+    they must be close on average with few outliers."""
+    e = row_errs(got, want)
+    if dtype is torch.float32:
+        assert float(e.max()) < 2e-4, (what, float(e.max()))
+    else:
+        assert float(e.mean()) < 0.05, (what, float(e.mean()))
+        assert float((e > 0.12).float().mean()) <= 0.1, (what, e)
 
 
 def replay(engine, requests: Dict[str, List[int]],

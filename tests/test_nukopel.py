@@ -1,0 +1,466 @@
+"""Nukopel on the CPU (fp32 torch ops): every mechanism against the plain
+oracle, then the served model — whole prompts, portions, token-by-token
+decoding, mixed batches, page/slot reuse, generation — against the oracle's
+whole-sequence logits. Configurations here are small and deliberately
+irregular (no two sizes equal, nothing a power of two where avoidable)."""
+import io
+import json
+import math
+import sys
+
+import pytest
+import torch
+
+from bee2bee_amd.models.spec import nukopel_spec
+from bee2bee_amd.ops import reference as ref
+from tests import nukopel_oracle as O
+from tests.nukopel_util import (assert_logits, chunk_schedule, make_engine,
+                                oracle_logits, random_tokens, rel_err, replay)
+
+F32 = torch.float32
+
+
+def i32(x):
+    return torch.tensor(x, dtype=torch.int32)
+
+
+# ------------------------------------------------------------- mechanisms
+
+def test_scalar_norms_match_oracle():
+    torch.manual_seed(0)
+    x = torch.randn(5, 37) * 4
+    y = torch.randn(5, 37)
+    g = torch.tensor(1.25)
+    want = O.scalar_norm(x.double(), g.double(), 1e-5)
+    assert torch.allclose(ref.scalar_rmsnorm(x, 1.25, 1e-5, F32).double(),
+                          want, atol=1e-5)
+    r = x.clone()
+    out = ref.add_scalar_rmsnorm(r, y, 0.5, 2.0, 1e-5, F32)
+    x2 = x.double() + O.scalar_norm(y.double(), torch.tensor(0.5).double(), 1e-5)
+    assert torch.allclose(r.double(), x2, atol=1e-5)
+    assert torch.allclose(out.double(),
+                          O.scalar_norm(x2, torch.tensor(2.0).double(), 1e-5),
+                          atol=1e-5)
+
+
+@pytest.mark.parametrize("taps", [1, 2, 3, 5])
+@pytest.mark.parametrize("cuts", [[12], [2, 2, 1, 7], [1] * 12, [5, 7]])
+def test_conv_portions_carry_state(taps, cuts):
+    torch.manual_seed(taps)
+    C, T = 9, 12
+    h = torch.randn(T, C)
+    w = torch.randn(C, taps)
+    want = h + O.causal_channel_conv(h, w)
+    # the slot starts full of NaN: nothing before position 0 may be read
+    state = torch.full((3, taps - 1, C), float("nan"))
+    got, at = [], 0
+    for n in cuts:
+        got.append(ref.canon_conv(h[at:at + n], w, state, i32([2]),
+                                  i32([0, n]), i32([0] * n),
+                                  i32(list(range(at, at + n)))))
+        at += n
+    assert torch.allclose(torch.cat(got), want, atol=1e-5)
+
+
+def test_conv_batch_of_unequal_chunks():
+    torch.manual_seed(1)
+    C, taps = 6, 4
+    w = torch.randn(C, taps)
+    seqs = [torch.randn(n, C) for n in (7, 3, 10)]
+    want = [s + O.causal_channel_conv(s, w) for s in seqs]
+    state = torch.full((4, taps - 1, C), float("nan"))
+    slots = i32([3, 0, 1])
+    # step 1: first portions 4, 1, 2; step 2: the rest
+    outs = [[], [], []]
+    at = [0, 0, 0]
+    for takes in ([4, 1, 2], [3, 2, 8]):
+        hs, cu, sidx, pos = [], [0], [], []
+        for b, n in enumerate(takes):
+            hs.append(seqs[b][at[b]:at[b] + n])
+            cu.append(cu[-1] + n)
+            sidx += [b] * n
+            pos += list(range(at[b], at[b] + n))
+        o = ref.canon_conv(torch.cat(hs), w, state, slots, i32(cu), i32(sidx),
+                           i32(pos))
+        for b, n in enumerate(takes):
+            outs[b].append(o[cu[b]:cu[b + 1]])
+            at[b] += n
+    for b in range(3):
+        assert torch.allclose(torch.cat(outs[b]), want[b], atol=1e-5)
+
+
+def test_rotation_and_latent_store():
+    torch.manual_seed(2)
+    T, H, R, C, dims = 6, 3, 10, 14, 6     # only 6 of the 10 dims rotate
+    pos = [0, 1, 2, 40, 41, 999]
+    q = torch.randn(T, H, R)
+    kv = torch.randn(T, C + R)
+    w = torch.rand(C) + 0.5
+    cos, sin = ref.rope_tables(1024, dims, 5000.0, "cpu")
+    cache = torch.zeros(4, 8, C + R)
+    slots = [3, 9, 31, 0, 17, 5]
+    q_in = q.clone()
+    ref.latent_rope_store(q, kv, w, 1e-5, C, dims, i32(pos), cos, sin, cache,
+                          i32(slots))
+    p = torch.tensor(pos)
+    assert torch.allclose(q.double(), O.rotate_pairs(q_in.double(), p, 5000.0,
+                                                     dims), atol=1e-4)
+    flat = cache.view(-1, C + R)[slots]
+    assert torch.allclose(flat[:, :C].double(), O.weighted_norm(
+        kv[:, :C].double(), w.double(), 1e-5), atol=1e-5)
+    assert torch.allclose(flat[:, C:].double(), O.rotate_pairs(
+        kv[:, C:].double(), p, 5000.0, dims), atol=1e-4)
+
+
+def _latent_setup(T, H, D, R, Dv, C, seed):
+    g = torch.Generator().manual_seed(seed)
+    c = torch.randn(T, C, generator=g)
+    k_rot = torch.randn(T, R, generator=g)
+    q = torch.randn(T, H, D + R, generator=g)
+    uk = torch.randn(H, D, C, generator=g) / math.sqrt(C)
+    uv = torch.randn(H, Dv, C, generator=g) / math.sqrt(C)
+    gate = torch.randn(T, H, generator=g)
+    return c, k_rot, q, uk, uv, gate
+
+
+def _latent_oracle(c, k_rot, q, uk, uv, gate, scale, window):
+    T, H = q.shape[:2]
+    D = uk.shape[1]
+    k = torch.cat([torch.einsum("hdc,tc->thd", uk, c),
+                   k_rot[:, None].expand(T, H, -1)], -1)
+    v = torch.einsum("hvc,tc->thv", uv, c)
+    o = O.windowed_softmax_attention(q.double(), k.double(), v.double(),
+                                     scale, window)
+    return o * torch.sigmoid(gate.double())[..., None]
+
+
+def _latent_framework(c, k_rot, q, uk, uv, gate, scale, window, cuts, bs=4):
+    """Absorbed-form op over a paged cache with scattered pages, fed in
+    portions; returns [T, H, Dv]."""
+    T, H = q.shape[:2]
+    D, C = uk.shape[1], uk.shape[2]
+    n_blocks = -(-T // bs) + 2
+    cache = torch.full((n_blocks, bs, C + k_rot.shape[1]), float("nan"))
+    bt = i32([[n_blocks - 1 - j for j in range(n_blocks)]])
+    outs, at = [], 0
+    for n in cuts:
+        pos = list(range(at, at + n))
+        for p in pos:
+            blk = int(bt[0, p // bs])
+            cache[blk, p % bs] = torch.cat([c[p], k_rot[p]])
+        q_abs = torch.einsum("thd,hdc->htc", q[at:at + n, :, :D], uk)
+        lat = ref.latent_attn(q_abs, q[at:at + n, :, D:], gate[at:at + n],
+                              cache, bt, i32(pos), i32([0] * n), i32([0, n]),
+                              window, scale)
+        outs.append(torch.einsum("htc,hvc->thv", lat, uv))
+        at += n
+    return torch.cat(outs)
+
+
+@pytest.mark.parametrize("window", [1, 2, 5, 100])
+@pytest.mark.parametrize("cuts", [[23], [3, 2, 9, 1, 1, 7], [1] * 23])
+def test_latent_attention_absorbed_equals_plain(window, cuts):
+    args = _latent_setup(23, 3, 6, 4, 5, 11, seed=window)
+    want = _latent_oracle(*args, 0.4, window)
+    got = _latent_framework(*args, 0.4, window, cuts)
+    assert torch.allclose(got.double(), want, atol=2e-5)
+
+
+@pytest.mark.parametrize("decoded", [False, True])
+def test_latent_window_edge_shows(decoded):
+    """One key is made to dominate: the last query must see it when it is
+    window-1 back, and must not when it is window back."""
+    T, window = 30, 8
+    for back, inside in ((window - 1, True), (window, False)):
+        c, k_rot, q, uk, uv, gate = _latent_setup(T, 2, 6, 4, 5, 11, seed=7)
+        j = T - 1 - back
+        k_rot[j] = 0
+        k_rot[j, 0] = 30.0
+        q[T - 1, :, 6:] = 0
+        q[T - 1, :, 6] = 30.0            # score 900 * scale on key j only
+        want = _latent_oracle(c, k_rot, q, uk, uv, gate, 0.4, window)
+        cuts = [T - 1, 1] if decoded else [T]
+        got = _latent_framework(c, k_rot, q, uk, uv, gate, 0.4, window, cuts)
+        assert torch.allclose(got.double(), want, atol=2e-5)
+        vj = torch.einsum("hvc,c->hv", uv, c[j]) * torch.sigmoid(
+            gate[T - 1])[:, None]
+        hit = torch.allclose(got[T - 1], vj, atol=1e-3)
+        assert hit == inside
+
+
+@pytest.mark.parametrize("cuts", [[150], [2, 63, 1, 64, 20], [70, 80],
+                                  [1] * 40 + [110]])
+def test_lightning_portions_match_recurrence(cuts):
+    torch.manual_seed(3)
+    T, H, D, Dv = 150, 3, 5, 7
+    q, k = torch.randn(T, H, D), torch.randn(T, H, D)
+    v = torch.randn(T, H, Dv)
+    decay = torch.tensor([0.3, 0.95, 1.0])
+    S = torch.zeros(H, D, Dv, dtype=torch.float64)
+    want = torch.zeros(T, H, Dv, dtype=torch.float64)
+    qs, ks, vs = (O.silu(t.double()) for t in (q, k, v))
+    for t in range(T):
+        S = decay.double()[:, None, None] * S + torch.einsum(
+            "hd,hv->hdv", ks[t], vs[t])
+        want[t] = torch.einsum("hdv,hd->hv", S, qs[t])
+    state = torch.full((2, H, D, Dv), float("nan"))
+    got, at = [], 0
+    for n in cuts:
+        got.append(ref.lightning_attn(q[at:at + n], k[at:at + n],
+                                      v[at:at + n], decay, state, i32([1]),
+                                      i32([0, n]),
+                                      i32(list(range(at, at + n)))))
+        at += n
+    got = torch.cat(got).view(T, H, Dv).double()
+    assert torch.allclose(got, want, rtol=1e-4, atol=1e-4)
+    assert torch.allclose(state[1].double(), S, rtol=1e-4, atol=1e-4)
+
+
+def test_lightning_far_token_is_remembered():
+    """With decay 1 a single early key/value pair must come back exactly,
+    hundreds of tokens and several portions later."""
+    T, D, Dv = 400, 4, 3
+    q = torch.full((T, 1, D), -20.0)     # silu(-20) ~ 0
+    k = torch.full((T, 1, D), -20.0)
+    v = torch.full((T, 1, Dv), -20.0)
+    k[5, 0, 2] = 3.0
+    v[5, 0] = torch.tensor([1.0, 2.0, 3.0])
+    q[T - 1, 0, 2] = 2.0
+    state = torch.zeros(1, 1, D, Dv)
+    outs, at = [], 0
+    for n in [100, 1, 2, 200, 96, 1]:
+        outs.append(ref.lightning_attn(q[at:at + n], k[at:at + n],
+                                       v[at:at + n], torch.tensor([1.0]),
+                                       state, i32([0]), i32([0, n]),
+                                       i32(list(range(at, at + n)))))
+        at += n
+    want = (O.silu(torch.tensor(2.0)) * O.silu(torch.tensor(3.0))
+            * O.silu(v[5, 0]))
+    assert torch.allclose(torch.cat(outs)[-1], want, atol=1e-4)
+
+
+def test_gated_norm_glu_and_router():
+    torch.manual_seed(4)
+    x, gate, w = torch.randn(4, 15), torch.randn(4, 15), torch.rand(15) + 0.5
+    want = O.weighted_norm(x.double(), w.double(), 1e-5) * torch.sigmoid(
+        gate.double())
+    assert torch.allclose(ref.gated_rmsnorm(x, w, gate, 1e-5, F32).double(),
+                          want, atol=1e-5)
+    h = torch.randn(6, 10) * 2
+    Wd = {"gate": torch.randn(7, 10), "up": torch.randn(7, 10),
+          "down": torch.randn(10, 7)}
+    gu = torch.cat([h @ Wd["gate"].T, h @ Wd["up"].T], -1)
+    got = ref.clamped_glu(gu, 1.1, 1.702) @ Wd["down"].T
+    want = O.expert(h.double(), {k: v.double() for k, v in Wd.items()}, "", 1.1)
+    assert torch.allclose(got.double(), want, atol=1e-4)
+    z = torch.randn(9, 6)
+    wts, idx = ref.moe_topk_gate(z, 3)
+    owts, oidx = O.route(z, torch.eye(6), 3)
+    assert torch.equal(idx.long(), oidx) and torch.allclose(wts, owts)
+
+
+@pytest.mark.parametrize("T", [3, 300])
+def test_moe_paths_match_oracle(tmp_path, T):
+    """The shared MoE executor (dense all-experts for small batches, sorted
+    per-expert for large ones) with the clamped GLU and fp32 routing."""
+    cfg = O.make_config(order=("lightning",), experts=6, top=3)
+    W = O.random_weights(cfg, seed=5)
+    eng = make_engine(tmp_path, cfg, W)
+    lw, f = eng.weights.layers[0], eng.spec.layer_specs[0].ffn
+    h = torch.randn(T, cfg["width"]).bfloat16().float()
+    got = eng.runner._moe_mlp(lw, h, ffn=f)
+    Wd = {k: v.double() for k, v in W.items()}
+    nf = dict(cfg["layers"][0]["mlp"], shared=None)
+    want = O.moe(h.double(), Wd, "l0.mlp.", nf)
+    assert torch.allclose(got.double(), want, atol=1e-4)
+
+
+# ------------------------------------------------------------ config/spec
+
+def test_config_is_read_not_assumed():
+    cfg = O.make_config(order=("latent_attention", "lightning"), taps=5,
+                        window=13, rot_dim=6, heads_la=5, heads_li=3,
+                        decay=(0.5, 0.6, 0.7), experts=7, top=4,
+                        emb_scale=2.5, eps=3e-4)
+    cfg["layers"][0]["mixer"]["rot"]["dims"] = 4
+    cfg["layers"][1]["mlp"] = None
+    s = nukopel_spec("x", cfg)
+    a, b = s.layer_specs
+    assert (s.canon_taps, s.embed_scale, s.rms_eps) == (5, 2.5, 3e-4)
+    assert (a.mixer.window, a.mixer.rot_dim, a.mixer.rope_dims,
+            a.mixer.heads) == (13, 6, 4, 5)
+    assert b.mixer.decay == (0.5, 0.6, 0.7) and b.ffn is None
+    assert (a.ffn.n_experts, a.ffn.top_k) == (7, 4)
+    assert s.is_hybrid and s.n_layers == 2
+
+
+# ------------------------------------------------------------ served model
+
+VARIANTS = {
+    "base": {},
+    "attn-first-no-shared": dict(order=("latent_attention", "lightning",
+                                        "latent_attention"), shared_ff=0),
+    "ones": dict(heads_la=1, heads_li=1, decay=(0.9,), top=1, taps=1,
+                 window=1, experts=2),
+    "equal-sizes": dict(dim=8, vdim=8, kv_rank=8, rot_dim=8, li_dim=8,
+                        li_vdim=8, ff=24, shared_ff=24, limit=1.0,
+                        shared_limit=1.0, window=16, taps=2,
+                        order=("lightning", "lightning", "latent_attention")),
+    "all-experts": dict(experts=3, top=3, window=64, taps=4, width=40,
+                        vocab=50),
+}
+
+
+def _cfg(name):
+    kw = dict(VARIANTS[name])
+    shared_off = kw.get("shared_ff") == 0
+    cfg = O.make_config(**kw)
+    if shared_off:
+        for l in cfg["layers"]:
+            l["mlp"]["shared"] = None
+    if name == "attn-first-no-shared":
+        cfg["layers"][1]["mlp"] = None
+        cfg["layers"][0]["mixer"]["rot"]["dims"] = 2
+    return cfg
+
+
+@pytest.mark.parametrize("name", list(VARIANTS))
+def test_served_model_matches_oracle(tmp_path, name):
+    cfg = _cfg(name)
+    W = O.random_weights(cfg, seed=11)
+    eng = make_engine(tmp_path, cfg, W)
+    toks = random_tokens(45, cfg["vocab"], 1)
+    want = oracle_logits(cfg, W, toks)
+    schedules = {
+        "whole": [[("a", 45)]],
+        "decode": [[("a", 9)]] + [[("a", 1)]] * 36,
+        "portions": chunk_schedule("a", 45, [2, 5, 1, 16, 3]),
+        "token-by-token": [[("a", 1)]] * 45,
+    }
+    for what, sched in schedules.items():
+        got = replay(eng, {"a": toks}, sched)["a"]
+        assert_logits(got, want, F32, what)
+    assert eng.kv.free_blocks == eng.kv.n_blocks - 1     # scratch page only
+
+
+def test_layer_residuals_match_oracle(tmp_path):
+    cfg = _cfg("base")
+    W = O.random_weights(cfg, seed=12)
+    eng = make_engine(tmp_path, cfg, W)
+    toks = random_tokens(19, cfg["vocab"], 2)
+    _, layers = O.forward(toks, W, cfg)
+    seen = []
+    eng.runner.layer_tap = lambda i, x: seen.append(x.clone())
+    eng.feed([("a", toks, [])], ["a"])
+    for i, x in enumerate(seen):
+        assert torch.allclose(x.double(), layers[i], atol=1e-3), i
+
+
+def test_mixed_batches_and_reuse(tmp_path):
+    """Unequal requests side by side (portions next to single tokens, a
+    request sitting out a step) equal each request alone; the pool is far
+    smaller than the sum of the requests, so pages and slots come back."""
+    cfg = _cfg("base")
+    W = O.random_weights(cfg, seed=13)
+    eng = make_engine(tmp_path, cfg, W, kv_blocks=7, block_size=8,
+                      max_batch=3)
+    lens = [21, 6, 30, 11, 17, 2, 26]
+    reqs = {f"r{i}": random_tokens(n, cfg["vocab"], 20 + i)
+            for i, n in enumerate(lens)}
+    sched = [
+        [("r0", 9), ("r1", 2)],
+        [("r0", 1), ("r1", 3), ("r2", 5)],
+        [("r0", 11), ("r2", 1)],                    # r1 sits out; r0 ends
+        [("r1", 1), ("r2", 2), ("r3", 11)],         # r1, r3 end
+        [("r2", 22), ("r4", 2)],                    # r2 ends
+        [("r4", 15), ("r5", 2), ("r6", 3)],         # r4, r5 end
+        [("r6", 1)], [("r6", 22)],
+    ]
+    got = replay(eng, reqs, sched)
+    for rid, toks in reqs.items():
+        assert_logits(got[rid], oracle_logits(cfg, W, toks), F32, rid)
+    assert eng.kv.free_blocks == eng.kv.n_blocks - 1
+    assert eng.kv.free_state_slots == eng.kv.n_state_slots - 1
+
+
+def test_long_decode_crosses_pages_and_windows(tmp_path):
+    cfg = _cfg("base")          # window 7, pages of 4 tokens here
+    W = O.random_weights(cfg, seed=14)
+    eng = make_engine(tmp_path, cfg, W, block_size=4, kv_blocks=50)
+    toks = random_tokens(140, cfg["vocab"], 3)
+    got = replay(eng, {"a": toks}, [[("a", 3)]] + [[("a", 1)]] * 137)["a"]
+    assert_logits(got, oracle_logits(cfg, W, toks), F32)
+
+
+def test_first_tokens_after_slot_reuse(tmp_path):
+    """A request that takes over a slot and pages another one just left must
+    not see anything of it in its first tokens."""
+    cfg = _cfg("base")
+    W = O.random_weights(cfg, seed=15)
+    eng = make_engine(tmp_path, cfg, W, max_batch=1, kv_blocks=3, block_size=16)
+    a, b = random_tokens(40, cfg["vocab"], 4), random_tokens(6, cfg["vocab"], 5)
+    replay(eng, {"a": a}, [[("a", 40)]])
+    for sched in ([[("b", 6)]], [[("b", 1)]] * 6, [[("b", 2)], [("b", 4)]]):
+        got = replay(eng, {"b": b}, sched)["b"]
+        assert_logits(got, oracle_logits(cfg, W, b), F32)
+
+
+def test_greedy_generation_through_scheduler(tmp_path):
+    """submit()/generate(): admission, chunked prompt prefill (budget of 7
+    tokens a step), batched decode of concurrent requests, retirement."""
+    cfg = _cfg("base")
+    W = O.random_weights(cfg, seed=16)
+    eng = make_engine(tmp_path, cfg, W, max_prefill_tokens=7)
+    try:
+        from bee2bee_amd.engine.engine import GenerationRequest
+        from bee2bee_amd.engine.sampler import SamplingParams
+
+        prompts = [random_tokens(n, cfg["vocab"], 30 + n) for n in (17, 3, 9)]
+        reqs = [eng.submit(GenerationRequest(
+            prompt_ids=list(p), max_new_tokens=10,
+            sampling=SamplingParams(greedy=True))) for p in prompts]
+        for r in reqs:
+            while r.done_ts is None:
+                r.out_queue.get(timeout=60)
+        for p, r in zip(prompts, reqs):
+            assert len(r.output_ids) == 10 and r.error is None
+            seq = list(p)
+            for tok in r.output_ids:
+                logits = oracle_logits(cfg, W, seq)[-1]
+                top2 = torch.topk(logits, 2).values
+                if float(top2[0] - top2[1]) > 1e-3:
+                    assert int(logits.argmax()) == tok
+                seq.append(tok)
+    finally:
+        eng.shutdown()
+
+
+def test_trace_replay_writes_wanted_logits(tmp_path, monkeypatch, capsys):
+    from bee2bee_amd.engine import trace
+
+    cfg = _cfg("base")
+    W = O.random_weights(cfg, seed=17)
+    O.save_checkpoint(str(tmp_path / "m"), cfg, W)
+    toks = random_tokens(12, cfg["vocab"], 6)
+    steps = [
+        {"step": 0, "entries": [{"id": "q", "tokens": toks[:7], "want": [0, 6]}],
+         "end": []},
+        {"step": 1, "entries": [{"id": "q", "tokens": toks[7:8], "want": []}],
+         "end": []},
+        {"step": 2, "entries": [{"id": "q", "tokens": toks[8:], "want": [3]}],
+         "end": ["q"]},
+    ]
+    monkeypatch.setattr(sys, "stdin", io.StringIO(
+        "\n".join(json.dumps(s) for s in steps) + "\n"))
+    out = tmp_path / "out"
+    assert trace.main(["--model", str(tmp_path / "m"), "--dtype", "float32",
+                       "--out", str(out), "--max-tokens", "64"]) == 0
+    assert capsys.readouterr().out.split() == ["done", "0", "done", "1",
+                                               "done", "2"]
+    import numpy as np
+
+    want = oracle_logits(cfg, W, toks)
+    a = torch.from_numpy(np.fromfile(out / "0.f32", dtype="<f4").reshape(2, -1))
+    c = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4").reshape(1, -1))
+    assert not (out / "1.f32").exists()
+    assert rel_err(a, want[[0, 6]]) < 2e-4 and rel_err(c, want[[11]]) < 2e-4
