@@ -422,7 +422,7 @@ class ModelWeights:
             tseed = (seed * 1000003 + zlib.crc32(name.encode())) % (2**31)
             gen = torch.Generator(device=self.device).manual_seed(tseed)
             shape, std = self._hybrid_shape(name)
-            t = torch.randn(*shape, generator=gen, dtype=torch.float32,
+            t = torch.randn(tuple(shape), generator=gen, dtype=torch.float32,
                             device=self.device)
             if std is None:               # gains / norm weights: around 1
                 return (1.0 + 0.1 * t).bfloat16()

@@ -7,6 +7,7 @@
 #include <ATen/hip/HIPContext.h>
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <optional>
 
 using torch::Tensor;
@@ -30,8 +31,8 @@ void launch_latent_rope_store(void*, long, long, int, const void*, long,
                               long, int, hipStream_t);
 int launch_latent_attn(const void*, const void*, long, long, const void*,
                        long, const void*, const int*, int, const int*,
-                       const int*, void*, int, int, int, int, int, int, float,
-                       int, hipStream_t);
+                       const int*, void*, float*, float*, int, int, int, int,
+                       int, int, int, float, int, hipStream_t);
 int launch_lightning(const void*, const void*, const void*, long,
                      const float*, float*, const int*, const int*, const int*,
                      float*, int, int, int, int, int, hipStream_t);
@@ -230,13 +231,27 @@ Tensor latent_attn(const Tensor& q_abs, const Tensor& q_rot,
     TORCH_CHECK(block_table.dim() == 2 && positions.numel() == Tn &&
                 seq_idx.numel() == Tn && window >= 1);
     Tensor out = torch::empty_like(q_abs);
+    // few rows (decode): split each row's keys over more workgroups until
+    // the chip has ~8 waves per SIMD, at least 32 keys per share
+    long splits = 8192 / std::max<long>(1, (long)Tn * H);
+    splits = std::min<long>({splits, 16, (window + 31) / 32});
+    splits = std::max<long>(splits, 1);
+    Tensor part_acc, part_ml;
+    float *pa = nullptr, *pm = nullptr;
+    if (splits > 1) {
+        auto f32 = q_abs.options().dtype(torch::kFloat32);
+        part_acc = torch::empty({splits, H, Tn, C}, f32);
+        part_ml = torch::empty({splits, H, Tn, 2}, f32);
+        pa = part_acc.data_ptr<float>();
+        pm = part_ml.data_ptr<float>();
+    }
     const int rc = launch_latent_attn(
         q_abs.data_ptr(), q_rot.data_ptr(), q_rot.stride(0), q_rot.stride(1),
         gate.data_ptr(), gate.stride(0), cache.data_ptr(),
         block_table.data_ptr<int>(), (int)block_table.size(1),
         positions.data_ptr<int>(), seq_idx.data_ptr<int>(), out.data_ptr(),
-        Tn, H, C, R, (int)cache.size(1), (int)window, (float)scale, c,
-        stream());
+        pa, pm, (int)splits, Tn, H, C, R, (int)cache.size(1), (int)window,
+        (float)scale, c, stream());
     TORCH_CHECK(rc == 0, "latent_attn: kv_rank + rot_dim must be <= 1024");
     return out;
 }

@@ -8,12 +8,15 @@
 // One wave per (token, head): lanes span the row's coordinates, keys are
 // walked four at a time with an online softmax; scores, weights and
 // accumulators are fp32. The same kernel serves prompt portions and decode
-// rows: every row carries its own position and sequence.
+// rows: every row carries its own position and sequence. When a step has
+// few rows (decode), the visible keys of each row are split over grid.z so
+// the chip is filled, and a second kernel merges the (max, sum, partial)
+// triples.
 //
 // lightning_attn: decayed linear attention S_t = lam_h S_(t-1) + k_t v_t^T,
 // o_t = S_t^T q_t with the state in fp32 registers. A workgroup owns a
-// 16-column slice of one (sequence, head) state — columns evolve
-// independently, which gives Dv/16-way parallelism per head on top of
+// 64-column slice of one (sequence, head) state — columns evolve
+// independently, which gives Dv/64-way parallelism per head on top of
 // sequences x heads — and walks the chunk's tokens in order.
 #include "common.h"
 
@@ -43,6 +46,8 @@ latent_attn_kernel(const T* __restrict__ q_abs,   // [H, Tn, C]
                    const int* __restrict__ positions,
                    const int* __restrict__ seq_idx,
                    T* __restrict__ out,           // [H, Tn, C]
+                   float* __restrict__ part_acc,  // [splits, H, Tn, C]
+                   float* __restrict__ part_ml,   // [splits, H, Tn, 2]
                    int Tn, int H, int C, int R, int bs, int window,
                    float scale) {
     const int t = blockIdx.x;
@@ -52,7 +57,16 @@ latent_attn_kernel(const T* __restrict__ q_abs,   // [H, Tn, C]
     const int Dk = C + R;
     const int p = positions[t];
     const int* bt = block_table + (long)seq_idx[t] * bt_stride;
-    const int lo = max(0, p - window + 1);
+    int lo = max(0, p - window + 1);
+    int last = p;
+    const int splits = gridDim.z;
+    if (splits > 1) {
+        // this workgroup's share of the visible keys (whole key groups)
+        int per = (p - lo + splits) / splits;
+        per = (per + LA_KEYS - 1) / LA_KEYS * LA_KEYS;
+        lo += blockIdx.z * per;
+        last = min(p, lo + per - 1);
+    }
 
     float qv[DPL], acc[DPL];
     const T* qa = q_abs + ((long)h * Tn + t) * C;
@@ -67,11 +81,11 @@ latent_attn_kernel(const T* __restrict__ q_abs,   // [H, Tn, C]
         acc[j] = 0.f;
     }
     float m = -INFINITY, l = 0.f;
-    for (int key = lo; key <= p; key += LA_KEYS) {
+    for (int key = lo; key <= last; key += LA_KEYS) {
         float kv[LA_KEYS][DPL], s[LA_KEYS];
 #pragma unroll
         for (int u = 0; u < LA_KEYS; ++u) {
-            const int kp = min(key + u, p);   // clamp: stay inside the pages
+            const int kp = min(key + u, last);  // clamp: stay inside the pages
             const T* row = cache + ((long)bt[kp / bs] * bs + kp % bs) * Dk;
             float d = 0.f;
 #pragma unroll
@@ -90,7 +104,7 @@ latent_attn_kernel(const T* __restrict__ q_abs,   // [H, Tn, C]
         float mn = m;
 #pragma unroll
         for (int u = 0; u < LA_KEYS; ++u) {
-            if (key + u > p) s[u] = -INFINITY;
+            if (key + u > last) s[u] = -INFINITY;
             mn = fmaxf(mn, s[u]);
         }
         const float a = expf(m - mn);
@@ -110,6 +124,20 @@ latent_attn_kernel(const T* __restrict__ q_abs,   // [H, Tn, C]
         }
         m = mn;
     }
+    if (splits > 1) {
+        // unnormalized partial + (max, sum); an empty share leaves l = 0
+        const long row = ((long)blockIdx.z * H + h) * Tn + t;
+#pragma unroll
+        for (int j = 0; j < DPL; ++j) {
+            const int c = lane + WAVE * j;
+            if (c < C) part_acc[row * C + c] = acc[j];
+        }
+        if (lane == 0) {
+            part_ml[row * 2] = m;
+            part_ml[row * 2 + 1] = l;
+        }
+        return;
+    }
     const float g = 1.f / (1.f + expf(-ldf(gate + (long)t * gate_tok + h)));
     const float r = g / l;
     T* o = out + ((long)h * Tn + t) * C;
@@ -120,13 +148,52 @@ latent_attn_kernel(const T* __restrict__ q_abs,   // [H, Tn, C]
     }
 }
 
+// merge the key-split partials of one (token, head): wave per row
+template <typename T>
+__global__ void __launch_bounds__(LA_WAVES * WAVE)
+latent_attn_combine_kernel(const float* __restrict__ part_acc,
+                           const float* __restrict__ part_ml,
+                           const T* __restrict__ gate, long gate_tok,
+                           T* __restrict__ out, int splits, int Tn, int H,
+                           int C) {
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x % WAVE;
+    const int h = blockIdx.y * LA_WAVES + threadIdx.x / WAVE;
+    if (h >= H) return;
+    float M = -INFINITY;
+    for (int z = 0; z < splits; ++z)
+        M = fmaxf(M, part_ml[(((long)z * H + h) * Tn + t) * 2]);
+    float L = 0.f;
+    for (int z = 0; z < splits; ++z) {
+        const long row = ((long)z * H + h) * Tn + t;
+        const float l = part_ml[row * 2 + 1];
+        if (l > 0.f) L += l * expf(part_ml[row * 2] - M);
+    }
+    const float g = 1.f / (1.f + expf(-ldf(gate + (long)t * gate_tok + h)));
+    T* o = out + ((long)h * Tn + t) * C;
+    for (int c = lane; c < C; c += WAVE) {
+        float a = 0.f;
+        for (int z = 0; z < splits; ++z) {
+            const long row = ((long)z * H + h) * Tn + t;
+            if (part_ml[row * 2 + 1] > 0.f)
+                a += part_acc[row * C + c] * expf(part_ml[row * 2] - M);
+        }
+        stf(o + c, a * g / L);
+    }
+}
+
 // ------------------------------------------------------------- lightning
-constexpr int LI_COLS = 16;    // state columns per workgroup
-constexpr int LI_GROUPS = 16;  // row groups (threads per column)
-constexpr int LI_TB = 4;       // tokens per reduction round
+constexpr int LI_COLS = 64;    // state columns per workgroup (one per lane)
+constexpr int LI_GROUPS = 4;   // row groups = waves; each owns D/4 state rows
+constexpr int LI_TB = 8;       // tokens staged per round
 
 DEV_INLINE float silu_f(float x) { return x / (1.f + expf(-x)); }
 
+// Workgroup = (sequence, head, 64-column slice of the state). Thread
+// (g, col) keeps rows [g*DPT, (g+1)*DPT) of column col in registers. Per
+// round of LI_TB tokens the block stages silu(q), silu(k) (all D rows) and
+// silu(v) (its columns) in LDS once — wave g then reads q/k as broadcasts —
+// and the four row groups' partial outputs are summed through LDS.
 template <typename T, int DPT>
 __global__ void __launch_bounds__(LI_COLS * LI_GROUPS)
 lightning_kernel(const T* __restrict__ q, const T* __restrict__ k,
@@ -138,12 +205,18 @@ lightning_kernel(const T* __restrict__ q, const T* __restrict__ k,
                  const int* __restrict__ positions,
                  float* __restrict__ out,          // [Tn, H * Dv]
                  int H, int D, int Dv) {
-    __shared__ float red[LI_TB][LI_GROUPS][LI_COLS + 1];
+    constexpr int DMAX = DPT * LI_GROUPS;
+    __shared__ float qs[LI_TB][DMAX];
+    __shared__ float ks[LI_TB][DMAX];
+    __shared__ float vs[LI_TB][LI_COLS];
+    __shared__ float red[LI_TB][LI_GROUPS][LI_COLS];
     const int b = blockIdx.x, h = blockIdx.y;
     const int lo = cu[b], hi = cu[b + 1];
     if (hi <= lo) return;
+    const int nth = LI_COLS * LI_GROUPS;
     const int g = threadIdx.x / LI_COLS, col = threadIdx.x % LI_COLS;
-    const int dv = blockIdx.z * LI_COLS + col;
+    const int c0 = blockIdx.z * LI_COLS;
+    const int dv = c0 + col;
     const bool live = dv < Dv;
     const int d0 = g * DPT;
     const float lam = decay[h];
@@ -157,33 +230,38 @@ lightning_kernel(const T* __restrict__ q, const T* __restrict__ k,
     }
     for (int t0 = lo; t0 < hi; t0 += LI_TB) {
         const int n = min(LI_TB, hi - t0);
+        for (int idx = threadIdx.x; idx < n * DMAX; idx += nth) {
+            const int tt = idx / DMAX, d = idx - tt * DMAX;
+            const long base = (long)(t0 + tt) * tok_stride + (long)h * D + d;
+            qs[tt][d] = d < D ? silu_f(ldf(q + base)) : 0.f;
+            ks[tt][d] = d < D ? silu_f(ldf(k + base)) : 0.f;
+        }
+        for (int idx = threadIdx.x; idx < n * LI_COLS; idx += nth) {
+            const int tt = idx / LI_COLS, c = idx - tt * LI_COLS;
+            vs[tt][c] = (c0 + c < Dv)
+                ? silu_f(ldf(v + (long)(t0 + tt) * tok_stride + (long)h * Dv + c0 + c))
+                : 0.f;
+        }
+        __syncthreads();
         for (int tt = 0; tt < n; ++tt) {
-            const long base = (long)(t0 + tt) * tok_stride;
-            const float vv = live ? silu_f(ldf(v + base + (long)h * Dv + dv)) : 0.f;
+            const float vv = vs[tt][col];
             float part = 0.f;
 #pragma unroll
             for (int i = 0; i < DPT; ++i) {
-                const int d = d0 + i;
-                if (d < D) {
-                    const float kk = silu_f(ldf(k + base + (long)h * D + d));
-                    const float qq = silu_f(ldf(q + base + (long)h * D + d));
-                    s[i] = lam * s[i] + kk * vv;
-                    part += s[i] * qq;
-                }
+                s[i] = lam * s[i] + ks[tt][d0 + i] * vv;
+                part += s[i] * qs[tt][d0 + i];
             }
             red[tt][g][col] = part;
         }
         __syncthreads();
-        if (threadIdx.x < n * LI_COLS) {
-            const int tt = threadIdx.x / LI_COLS, c2 = threadIdx.x % LI_COLS;
-            const int dv2 = blockIdx.z * LI_COLS + c2;
+        for (int idx = threadIdx.x; idx < n * LI_COLS; idx += nth) {
+            const int tt = idx / LI_COLS, c = idx - tt * LI_COLS;
             float o = 0.f;
 #pragma unroll
-            for (int gg = 0; gg < LI_GROUPS; ++gg) o += red[tt][gg][c2];
-            if (dv2 < Dv)
-                out[(long)(t0 + tt) * H * Dv + (long)h * Dv + dv2] = o;
+            for (int gg = 0; gg < LI_GROUPS; ++gg) o += red[tt][gg][c];
+            if (c0 + c < Dv)
+                out[(long)(t0 + tt) * H * Dv + (long)h * Dv + c0 + c] = o;
         }
-        __syncthreads();
     }
     if (live) {
 #pragma unroll
@@ -201,8 +279,8 @@ lightning_kernel(const T* __restrict__ q, const T* __restrict__ k,
         latent_attn_kernel<TT, N><<<grid, LA_WAVES * WAVE, 0, s>>>(           \
             (const TT*)q_abs, (const TT*)q_rot, qr_tok, qr_head,              \
             (const TT*)gate, gate_tok, (const TT*)cache, block_table,         \
-            bt_stride, positions, seq_idx, (TT*)out, Tn, H, C, R, bs, window, \
-            scale);                                                           \
+            bt_stride, positions, seq_idx, (TT*)out, part_acc, part_ml, Tn,   \
+            H, C, R, bs, window, scale);                                      \
         break;
 
 template <typename TT>
@@ -211,18 +289,26 @@ static int latent_attn_dispatch(const void* q_abs, const void* q_rot,
                                 long gate_tok, const void* cache,
                                 const int* block_table, int bt_stride,
                                 const int* positions, const int* seq_idx,
-                                void* out, int Tn, int H, int C, int R, int bs,
-                                int window, float scale, hipStream_t s) {
+                                void* out, float* part_acc, float* part_ml,
+                                int splits, int Tn, int H, int C, int R,
+                                int bs, int window, float scale,
+                                hipStream_t s) {
     const int need = (C + R + WAVE - 1) / WAVE;
     const int sizes[] = {1, 2, 3, 4, 6, 9, 12, 16};
     int dpl = 0;
     for (int z : sizes)
         if (z >= need) { dpl = z; break; }
     if (!dpl) return 1;
-    const dim3 grid(Tn, (H + LA_WAVES - 1) / LA_WAVES);
+    const dim3 grid(Tn, (H + LA_WAVES - 1) / LA_WAVES, splits);
     switch (dpl) {
         LA_CASE(1) LA_CASE(2) LA_CASE(3) LA_CASE(4) LA_CASE(6) LA_CASE(9)
         LA_CASE(12) LA_CASE(16)
+    }
+    if (splits > 1) {
+        const dim3 g2(Tn, (H + LA_WAVES - 1) / LA_WAVES);
+        latent_attn_combine_kernel<TT><<<g2, LA_WAVES * WAVE, 0, s>>>(
+            part_acc, part_ml, (const TT*)gate, gate_tok, (TT*)out, splits,
+            Tn, H, C);
     }
     return 0;
 }
@@ -233,17 +319,20 @@ extern "C" int launch_latent_attn(const void* q_abs, const void* q_rot,
                                   long gate_tok, const void* cache,
                                   const int* block_table, int bt_stride,
                                   const int* positions, const int* seq_idx,
-                                  void* out, int Tn, int H, int C, int R,
+                                  void* out, float* part_acc, float* part_ml,
+                                  int splits, int Tn, int H, int C, int R,
                                   int bs, int window, float scale, int f32,
                                   hipStream_t s) {
     if (Tn == 0) return 0;
     if (f32)
         return latent_attn_dispatch<float>(
             q_abs, q_rot, qr_tok, qr_head, gate, gate_tok, cache, block_table,
-            bt_stride, positions, seq_idx, out, Tn, H, C, R, bs, window, scale, s);
+            bt_stride, positions, seq_idx, out, part_acc, part_ml, splits, Tn,
+            H, C, R, bs, window, scale, s);
     return latent_attn_dispatch<unsigned short>(
         q_abs, q_rot, qr_tok, qr_head, gate, gate_tok, cache, block_table,
-        bt_stride, positions, seq_idx, out, Tn, H, C, R, bs, window, scale, s);
+        bt_stride, positions, seq_idx, out, part_acc, part_ml, splits, Tn, H,
+        C, R, bs, window, scale, s);
 }
 
 #define LI_CASE(N)                                                            \
@@ -260,13 +349,13 @@ static int lightning_dispatch(const void* q, const void* k, const void* v,
                               const int* cu, const int* positions, float* out,
                               int B, int H, int D, int Dv, hipStream_t s) {
     const int need = (D + LI_GROUPS - 1) / LI_GROUPS;
-    const int sizes[] = {1, 2, 4, 8, 16};
+    const int sizes[] = {2, 8, 16, 32, 64};
     int dpt = 0;
     for (int z : sizes)
         if (z >= need) { dpt = z; break; }
     if (!dpt) return 1;
     const dim3 grid(B, H, (Dv + LI_COLS - 1) / LI_COLS);
-    switch (dpt) { LI_CASE(1) LI_CASE(2) LI_CASE(4) LI_CASE(8) LI_CASE(16) }
+    switch (dpt) { LI_CASE(2) LI_CASE(8) LI_CASE(16) LI_CASE(32) LI_CASE(64) }
     return 0;
 }
 

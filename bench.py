@@ -26,6 +26,94 @@ sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 import torch
 
 
+# layer sizes for --compare-hybrid: (width, heads, layers, experts, ff)
+HYBRID_SIZES = {
+    "s": dict(width=1024, heads=8, layers=4, experts=8, ff=512),
+    "m": dict(width=2048, heads=16, layers=4, experts=8, ff=1024),
+    "l": dict(width=4096, heads=32, layers=4, experts=8, ff=2048),
+}
+
+
+def compare_hybrid(args) -> None:
+    """Prefill and decode throughput of a Nukopel stack (3 linear-attention
+    layers per latent-attention layer, routed + shared experts) and of the
+    closest dense-attention stack the framework serves (GQA attention,
+    routed experts) at the same width, depth and expert sizes. Random
+    weights, synthetic prompts, one GPU."""
+    from bee2bee_amd.engine.engine import InferenceEngine
+    from bee2bee_amd.models.hybrid import nukopel_layers
+    from bee2bee_amd.models.spec import ModelSpec, hybrid_spec
+
+    on_gpu = torch.cuda.is_available()
+    device = "cuda:0" if on_gpu else "cpu"
+    vocab, head_dim = 32000, 128
+    p_batch, p_len = 8, (2048 if on_gpu else 64)
+    d_batch, d_len = (64 if on_gpu else 4), (1024 if on_gpu else 32)
+    budget = args.warmup + args.steps + 4
+
+    def sync() -> None:
+        if on_gpu:
+            torch.cuda.synchronize()
+
+    for size in args.compare_hybrid.split(","):
+        z = HYBRID_SIZES[size.strip()]
+        W, H, L = z["width"], z["heads"], z["layers"]
+        nk = hybrid_spec(
+            f"nukopel-{size}", vocab, W,
+            nukopel_layers(L, W, heads=H, dim=head_dim, rot_dim=64,
+                           vdim=head_dim, kv_rank=512, window=4096,
+                           li_heads=H, li_dim=head_dim, li_vdim=head_dim,
+                           experts=z["experts"], top_k=2, ff=z["ff"],
+                           shared_ff=z["ff"]),
+            eps=1e-6, embed_scale=1.0, canon_taps=4, max_seq_len=8192)
+        dense = ModelSpec(
+            name=f"gqa-moe-{size}", vocab_size=vocab, hidden_size=W,
+            intermediate_size=z["ff"], n_layers=L, n_heads=H,
+            n_kv_heads=max(1, H // 4), head_dim=head_dim, rope_theta=1e6,
+            max_seq_len=8192, n_experts=z["experts"], top_k_experts=2)
+        for spec in (nk, dense):
+            engine = InferenceEngine(
+                spec, device=device, max_batch=max(d_batch, p_batch),
+                max_seq_len=max(p_len, d_len) + budget + 8,
+                use_graphs=(not args.no_graphs) and on_gpu,
+                max_prefill_tokens=8192, seed=1234)
+            times = []
+            for _ in range(2):           # first pass is the warmup
+                sync()
+                t0 = time.perf_counter()
+                ids = engine.bench_prefill(p_batch, p_len, max_new=1)
+                sync()
+                times.append(time.perf_counter() - t0)
+                for sid in ids:
+                    engine.kv.free_seq(sid)
+            prefill_tps = p_batch * p_len / times[-1]
+            engine.bench_setup(d_batch, d_len, budget)
+            for _ in range(args.warmup):
+                engine.bench_step()
+            sync()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                engine.bench_step()
+            sync()
+            dt = time.perf_counter() - t0
+            print(json.dumps({
+                "compare": "hybrid-vs-dense", "size": size, "model": spec.name,
+                "params_m": round(spec.n_params() / 1e6, 1),
+                "prefill_tokens_per_s": round(prefill_tps, 1),
+                "prefill_shape": [p_batch, p_len],
+                "decode_tokens_per_s": round(d_batch * args.steps / dt, 1),
+                "decode_ms_per_step": round(dt / args.steps * 1e3, 3),
+                "decode_shape": [d_batch, d_len],
+                "decode_graphs": engine.graphs is not None,
+                "dtype": "bf16" if on_gpu else "fp32-cpu",
+                "data": "synthetic",
+            }), flush=True)
+            engine.shutdown()
+            del engine
+            if on_gpu:
+                torch.cuda.empty_cache()
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -40,6 +128,12 @@ def main() -> None:
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--no-tunableop", action="store_true",
                     help="skip hipBLASLt algorithm tuning")
+    ap.add_argument("--compare-hybrid", default=None, metavar="SIZES",
+                    help="instead of the headline run: prefill and decode "
+                         "throughput of the Nukopel hybrid stack beside a "
+                         "dense-attention MoE stack of equal width, depth "
+                         "and expert sizes, at the comma-separated sizes "
+                         "(s, m, l); one JSON line per size and model")
     ap.add_argument("--preflight", action="store_true",
                     help="run the scale-run preflight checks (RCCL self-"
                          "test, master endpoint, env, rank wiring) and exit")
@@ -53,6 +147,10 @@ def main() -> None:
         report = run_preflight(args.gpus, tune_dir)
         print(json.dumps(report), flush=True)
         sys.exit(0 if report["preflight"] == "ok" else 1)
+
+    if args.compare_hybrid:
+        compare_hybrid(args)
+        return
 
     from bee2bee_amd.models.spec import resolve_spec
 
