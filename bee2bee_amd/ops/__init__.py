@@ -291,7 +291,7 @@ def latent_attn(q_abs, q_rot, gate, cache, block_table, positions, seq_idx,
     if _use_hip(q_abs):
         return require_hip().latent_attn(q_abs, q_rot, gate, cache,
                                          block_table, positions, seq_idx,
-                                         window, scale, max_qlen)
+                                         cu_seqlens, window, scale, max_qlen)
     return reference.latent_attn(q_abs, q_rot, gate, cache, block_table,
                                  positions, seq_idx, cu_seqlens, window, scale)
 

@@ -33,6 +33,10 @@ int launch_latent_attn(const void*, const void*, long, long, const void*,
                        long, const void*, const int*, int, const int*,
                        const int*, void*, float*, float*, int, int, int, int,
                        int, int, int, float, int, hipStream_t);
+int launch_latent_attn_mfma(const void*, const void*, long, long, const void*,
+                            long, const void*, const int*, int, const int*,
+                            const int*, void*, int, int, int, int, int, int,
+                            int, int, float, hipStream_t);
 int launch_lightning(const void*, const void*, const void*, long,
                      const float*, float*, const int*, const int*, const int*,
                      float*, int, int, int, int, int, hipStream_t);
@@ -209,9 +213,10 @@ void latent_rope_store(Tensor& q_rot, const Tensor& kv, const Tensor& kv_norm,
 Tensor latent_attn(const Tensor& q_abs, const Tensor& q_rot,
                    const Tensor& gate, const Tensor& cache,
                    const Tensor& block_table, const Tensor& positions,
-                   const Tensor& seq_idx, int64_t window, double scale,
-                   int64_t max_qlen) {
+                   const Tensor& seq_idx, const Tensor& cu, int64_t window,
+                   double scale, int64_t max_qlen) {
     const int c = act_code(q_abs, "q_abs");
+    check_i32(cu, "cu_seqlens");
     check_i32(block_table, "block_table");
     check_i32(positions, "positions");
     check_i32(seq_idx, "seq_idx");
@@ -231,6 +236,20 @@ Tensor latent_attn(const Tensor& q_abs, const Tensor& q_rot,
     TORCH_CHECK(block_table.dim() == 2 && positions.numel() == Tn &&
                 seq_idx.numel() == Tn && window >= 1);
     Tensor out = torch::empty_like(q_abs);
+    // prompt portions in bf16 run on the matrix cores (16-query tiles);
+    // steps of single tokens, fp32, and uncovered shapes take the generic
+    // kernel below
+    if (c == 0 && max_qlen >= 16) {
+        const int rc = launch_latent_attn_mfma(
+            q_abs.data_ptr(), q_rot.data_ptr(), q_rot.stride(0),
+            q_rot.stride(1), gate.data_ptr(), gate.stride(0),
+            cache.data_ptr(), block_table.data_ptr<int>(),
+            (int)block_table.size(1), cu.data_ptr<int>(),
+            positions.data_ptr<int>(), out.data_ptr(), Tn,
+            (int)cu.numel() - 1, (int)max_qlen, H, C, R, (int)cache.size(1),
+            (int)window, (float)scale, stream());
+        if (rc == 0) return out;
+    }
     // few rows (decode): split each row's keys over more workgroups until
     // the chip has ~8 waves per SIMD, at least 32 keys per share
     long splits = 8192 / std::max<long>(1, (long)Tn * H);

@@ -148,6 +148,198 @@ latent_attn_kernel(const T* __restrict__ q_abs,   // [H, Tn, C]
     }
 }
 
+
+// ------------------------------------------------- latent attention, MFMA
+// bf16 prompt portions: workgroup = 16 consecutive queries of one sequence
+// x 4 heads (one wave per head; all heads share the cached rows, so one
+// staged key tile serves 64 query rows). Per 32-key tile: S = Q K^T on
+// v_mfma_f32_16x16x32_bf16 (fp32 scores, scaled in fp32), window + causal
+// mask, online softmax in fp32, then O += P K[:, :C] with the fp32 weights
+// carried as a bf16 pair (hi + lo, two MFMAs) so they keep ~16 mantissa
+// bits. Fragment maps (gfx950): A 16x32: lane -> row l&15, k (l>>4)*8+e;
+// B 32x16: lane -> col l&15, k (l>>4)*8+e; C 16x16: col l&15, rows
+// (l>>4)*4+r.
+constexpr int LM_TN = 32;
+constexpr int LM_PAD = 8;
+
+template <int KSTEPS>
+__global__ void __launch_bounds__(256)
+latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
+                        const unsigned short* __restrict__ q_rot, long qr_tok,
+                        long qr_head, const unsigned short* __restrict__ gate,
+                        long gate_tok,
+                        const unsigned short* __restrict__ cache,
+                        const int* __restrict__ block_table, int bt_stride,
+                        const int* __restrict__ cu,
+                        const int* __restrict__ positions,
+                        unsigned short* __restrict__ out, int Tn, int H, int C,
+                        int R, int bs, int window, float scale) {
+    constexpr int DKP = KSTEPS * 32;
+    constexpr int KS = DKP + LM_PAD;       // key tile row stride
+    constexpr int PS = LM_TN + LM_PAD;     // weight tile row stride
+    __shared__ __attribute__((aligned(16))) unsigned short k_s[LM_TN * KS];
+    __shared__ __attribute__((aligned(16))) unsigned short p_hi[64 * PS];
+    __shared__ __attribute__((aligned(16))) unsigned short p_lo[64 * PS];
+
+    const int seq = blockIdx.z;
+    const int s0 = cu[seq];
+    const int QL = cu[seq + 1] - s0;
+    const int q0 = blockIdx.x * 16;
+    if (q0 >= QL) return;
+    const int tid = threadIdx.x, lane = tid % WAVE, wid = tid / WAVE;
+    const int lg = lane >> 4, li = lane & 15;
+    const int h = blockIdx.y * 4 + wid;
+    const bool head_ok = h < H;
+    const int Dk = C + R;
+    const int hist = positions[s0];
+    const int* bt = block_table + (long)seq * bt_stride;
+
+    bf16x8 a_q[KSTEPS];
+    {
+        const int row = q0 + li;
+        const bool ok = head_ok && row < QL;
+        const unsigned short* qa = q_abs + ((long)h * Tn + s0 + row) * C;
+        const unsigned short* qr = q_rot + (long)(s0 + row) * qr_tok +
+                                   (long)h * qr_head;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            short8 raw;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int c = ks * 32 + lg * 8 + e;
+                unsigned short v = 0;
+                if (ok && c < C) v = qa[c];
+                else if (ok && c < Dk) v = qr[c - C];
+                raw[e] = (short)v;
+            }
+            a_q[ks] = __builtin_bit_cast(bf16x8, raw);
+        }
+    }
+    float m_run[4], l_run[4];
+    f32x4 o_acc[KSTEPS * 2];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) { m_run[r] = -1e30f; l_run[r] = 0.f; }
+#pragma unroll
+    for (int nb = 0; nb < KSTEPS * 2; ++nb) o_acc[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int last_row = min(q0 + 15, QL - 1);
+    const int kv_lo = max(0, hist + q0 - window + 1);
+    const int kv_end = hist + last_row + 1;
+
+    for (int kb = kv_lo; kb < kv_end; kb += LM_TN) {
+        __syncthreads();   // previous tile's reads of k_s are done
+        constexpr int UNITS = DKP / 8;
+        for (int i = tid; i < LM_TN * UNITS; i += 256) {
+            const int key = i / UNITS, d = (i - key * UNITS) * 8;
+            const int gk = kb + key;
+            short8 raw = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (gk < kv_end && d < Dk)
+                raw = *reinterpret_cast<const short8*>(
+                    cache + ((long)bt[gk / bs] * bs + gk % bs) * Dk + d);
+            *reinterpret_cast<short8*>(k_s + key * KS + d) = raw;
+        }
+        __syncthreads();
+
+        f32x4 sfrag[LM_TN / 16];
+#pragma unroll
+        for (int f = 0; f < LM_TN / 16; ++f) {
+            f32x4 acc{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) {
+                const bf16x8 bk = *reinterpret_cast<const bf16x8*>(
+                    k_s + (f * 16 + li) * KS + ks * 32 + lg * 8);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_q[ks], bk, acc,
+                                                              0, 0, 0);
+            }
+            sfrag[f] = acc;
+        }
+        float pmax[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) pmax[r] = -1e30f;
+#pragma unroll
+        for (int f = 0; f < LM_TN / 16; ++f) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int qrow = q0 + lg * 4 + r;
+                const int back = hist + qrow - (kb + f * 16 + li);
+                const bool vis = qrow < QL && back >= 0 && back < window;
+                sfrag[f][r] = vis ? sfrag[f][r] * scale : -1e30f;
+                pmax[r] = fmaxf(pmax[r], sfrag[f][r]);
+            }
+        }
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                pmax[r] = fmaxf(pmax[r], __shfl_xor(pmax[r], off));
+        float alpha[4], psum[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float mn = fmaxf(m_run[r], pmax[r]);
+            alpha[r] = expf(m_run[r] - mn);
+            m_run[r] = mn;
+            psum[r] = 0.f;
+        }
+#pragma unroll
+        for (int f = 0; f < LM_TN / 16; ++f) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float pv = expf(sfrag[f][r] - m_run[r]);
+                if (sfrag[f][r] <= -1e29f) pv = 0.f;
+                psum[r] += pv;
+                const unsigned short hi = f2bf(pv);
+                const int at = (wid * 16 + lg * 4 + r) * PS + f * 16 + li;
+                p_hi[at] = hi;
+                p_lo[at] = f2bf(pv - bf2f(hi));
+            }
+        }
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) psum[r] += __shfl_xor(psum[r], off);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) l_run[r] = l_run[r] * alpha[r] + psum[r];
+#pragma unroll
+        for (int nb = 0; nb < KSTEPS * 2; ++nb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o_acc[nb][r] *= alpha[r];
+        __syncthreads();   // weight tile visible to the wave's other lanes
+        const bf16x8 a_hi = *reinterpret_cast<const bf16x8*>(
+            p_hi + (wid * 16 + li) * PS + lg * 8);
+        const bf16x8 a_lo = *reinterpret_cast<const bf16x8*>(
+            p_lo + (wid * 16 + li) * PS + lg * 8);
+#pragma unroll
+        for (int nb = 0; nb < KSTEPS * 2; ++nb) {
+            if (nb * 16 < C) {
+                short8 raw;
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    raw[e] = (short)k_s[(lg * 8 + e) * KS + nb * 16 + li];
+                const bf16x8 bv = __builtin_bit_cast(bf16x8, raw);
+                o_acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    a_hi, bv, o_acc[nb], 0, 0, 0);
+                o_acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    a_lo, bv, o_acc[nb], 0, 0, 0);
+            }
+        }
+    }
+    if (!head_ok) return;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int qrow = q0 + lg * 4 + r;
+        if (qrow >= QL) continue;
+        const float g = 1.f / (1.f + expf(-bf2f(
+            gate[(long)(s0 + qrow) * gate_tok + h])));
+        const float inv = l_run[r] > 0.f ? g / l_run[r] : 0.f;
+        unsigned short* orow = out + ((long)h * Tn + s0 + qrow) * C;
+#pragma unroll
+        for (int nb = 0; nb < KSTEPS * 2; ++nb) {
+            const int c = nb * 16 + li;
+            if (c < C) orow[c] = f2bf(o_acc[nb][r] * inv);
+        }
+    }
+}
+
 // merge the key-split partials of one (token, head): wave per row
 template <typename T>
 __global__ void __launch_bounds__(LA_WAVES * WAVE)
@@ -333,6 +525,34 @@ extern "C" int launch_latent_attn(const void* q_abs, const void* q_rot,
         q_abs, q_rot, qr_tok, qr_head, gate, gate_tok, cache, block_table,
         bt_stride, positions, seq_idx, out, part_acc, part_ml, splits, Tn, H,
         C, R, bs, window, scale, s);
+}
+
+#define LM_CASE(N)                                                            \
+    latent_attn_mfma_kernel<N><<<grid, 256, 0, s>>>(                          \
+        (const unsigned short*)q_abs, (const unsigned short*)q_rot, qr_tok,   \
+        qr_head, (const unsigned short*)gate, gate_tok,                       \
+        (const unsigned short*)cache, block_table, bt_stride, cu, positions,  \
+        (unsigned short*)out, Tn, H, C, R, bs, window, scale)
+
+// bf16 prompt portions on the matrix cores. Returns nonzero when the shape
+// is not covered (row width not a multiple of 8 or above 576) and the
+// caller should use the generic kernel.
+extern "C" int launch_latent_attn_mfma(
+    const void* q_abs, const void* q_rot, long qr_tok, long qr_head,
+    const void* gate, long gate_tok, const void* cache,
+    const int* block_table, int bt_stride, const int* cu,
+    const int* positions, void* out, int Tn, int B, int max_qlen, int H,
+    int C, int R, int bs, int window, float scale, hipStream_t s) {
+    const int Dk = C + R;
+    if (Dk % 8 != 0 || Dk > 576) return 1;
+    if (Tn == 0 || B == 0) return 0;
+    const dim3 grid((max_qlen + 15) / 16, (H + 3) / 4, B);
+    const int ksteps = (Dk + 31) / 32;
+    if (ksteps <= 4) LM_CASE(4);
+    else if (ksteps <= 8) LM_CASE(8);
+    else if (ksteps <= 12) LM_CASE(12);
+    else LM_CASE(18);
+    return 0;
 }
 
 #define LI_CASE(N)                                                            \
