@@ -35,8 +35,9 @@ int launch_latent_attn(const void*, const void*, long, long, const void*,
                        int, int, int, float, int, hipStream_t);
 int launch_latent_attn_mfma(const void*, const void*, long, long, const void*,
                             long, const void*, const int*, int, const int*,
-                            const int*, void*, int, int, int, int, int, int,
-                            int, int, float, hipStream_t);
+                            const int*, const int*, void*, float*, float*,
+                            int, int, int, int, int, int, int, int, int,
+                            float, hipStream_t);
 int launch_lightning(const void*, const void*, const void*, long,
                      const float*, float*, const int*, const int*, const int*,
                      float*, int, int, int, int, int, hipStream_t);
@@ -236,34 +237,45 @@ Tensor latent_attn(const Tensor& q_abs, const Tensor& q_rot,
     TORCH_CHECK(block_table.dim() == 2 && positions.numel() == Tn &&
                 seq_idx.numel() == Tn && window >= 1);
     Tensor out = torch::empty_like(q_abs);
-    // prompt portions in bf16 run on the matrix cores (16-query tiles);
-    // steps of single tokens, fp32, and uncovered shapes take the generic
-    // kernel below
-    if (c == 0 && max_qlen >= 16) {
+    auto f32opt = q_abs.options().dtype(torch::kFloat32);
+    Tensor part_acc, part_ml;
+    float *pa = nullptr, *pm = nullptr;
+    auto alloc_parts = [&](long n) {
+        part_acc = torch::empty({n, H, Tn, C}, f32opt);
+        part_ml = torch::empty({n, H, Tn, 2}, f32opt);
+        pa = part_acc.data_ptr<float>();
+        pm = part_ml.data_ptr<float>();
+    };
+    // bf16 prompt portions (16-query tiles) and pure decode steps (16-head
+    // tiles, keys split until ~1024 workgroups) run on the matrix cores;
+    // fp32, short mixed steps and uncovered shapes take the generic kernel
+    if (c == 0 && (max_qlen >= 16 || max_qlen == 1) && (C + R) % 8 == 0 &&
+        C + R <= 576) {
+        long sp = 1;
+        if (max_qlen == 1) {
+            sp = 1024 / std::max<long>(1, (long)Tn * ((H + 15) / 16));
+            sp = std::max<long>(1, std::min<long>({sp, 16, (window + 63) / 64}));
+            if (sp > 1) alloc_parts(sp);
+        }
         const int rc = launch_latent_attn_mfma(
             q_abs.data_ptr(), q_rot.data_ptr(), q_rot.stride(0),
             q_rot.stride(1), gate.data_ptr(), gate.stride(0),
             cache.data_ptr(), block_table.data_ptr<int>(),
             (int)block_table.size(1), cu.data_ptr<int>(),
-            positions.data_ptr<int>(), out.data_ptr(), Tn,
-            (int)cu.numel() - 1, (int)max_qlen, H, C, R, (int)cache.size(1),
-            (int)window, (float)scale, stream());
-        if (rc == 0) return out;
+            positions.data_ptr<int>(), seq_idx.data_ptr<int>(),
+            out.data_ptr(), pa, pm, (int)sp, Tn, (int)cu.numel() - 1,
+            (int)max_qlen, H, C, R, (int)cache.size(1), (int)window,
+            (float)scale, stream());
+        TORCH_CHECK(rc == 0, "latent_attn: matrix-core path refused a shape "
+                             "its guard admitted");
+        return out;
     }
-    // few rows (decode): split each row's keys over more workgroups until
-    // the chip has ~8 waves per SIMD, at least 32 keys per share
+    // few rows: split each row's keys over more workgroups until the chip
+    // has ~8 waves per SIMD, at least 32 keys per share
     long splits = 8192 / std::max<long>(1, (long)Tn * H);
     splits = std::min<long>({splits, 16, (window + 31) / 32});
     splits = std::max<long>(splits, 1);
-    Tensor part_acc, part_ml;
-    float *pa = nullptr, *pm = nullptr;
-    if (splits > 1) {
-        auto f32 = q_abs.options().dtype(torch::kFloat32);
-        part_acc = torch::empty({splits, H, Tn, C}, f32);
-        part_ml = torch::empty({splits, H, Tn, 2}, f32);
-        pa = part_acc.data_ptr<float>();
-        pm = part_ml.data_ptr<float>();
-    }
+    if (splits > 1) alloc_parts(splits);
     const int rc = launch_latent_attn(
         q_abs.data_ptr(), q_rot.data_ptr(), q_rot.stride(0), q_rot.stride(1),
         gate.data_ptr(), gate.stride(0), cache.data_ptr(),

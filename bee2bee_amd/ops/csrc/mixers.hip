@@ -162,8 +162,8 @@ latent_attn_kernel(const T* __restrict__ q_abs,   // [H, Tn, C]
 constexpr int LM_TN = 32;
 constexpr int LM_PAD = 8;
 
-template <int KSTEPS>
-__global__ void __launch_bounds__(256)
+template <int KSTEPS, bool DECODE>
+__global__ void __launch_bounds__(DECODE ? 64 : 256)
 latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
                         const unsigned short* __restrict__ q_rot, long qr_tok,
                         long qr_head, const unsigned short* __restrict__ gate,
@@ -172,7 +172,10 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
                         const int* __restrict__ block_table, int bt_stride,
                         const int* __restrict__ cu,
                         const int* __restrict__ positions,
-                        unsigned short* __restrict__ out, int Tn, int H, int C,
+                        const int* __restrict__ seq_idx,
+                        unsigned short* __restrict__ out,
+                        float* __restrict__ part_acc,
+                        float* __restrict__ part_ml, int Tn, int H, int C,
                         int R, int bs, int window, float scale) {
     constexpr int DKP = KSTEPS * 32;
     constexpr int KS = DKP + LM_PAD;       // key tile row stride
@@ -181,14 +184,19 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
     __shared__ __attribute__((aligned(16))) unsigned short p_hi[64 * PS];
     __shared__ __attribute__((aligned(16))) unsigned short p_lo[64 * PS];
 
-    const int seq = blockIdx.z;
-    const int s0 = cu[seq];
-    const int QL = cu[seq + 1] - s0;
-    const int q0 = blockIdx.x * 16;
+    // PREFILL: rows = 16 queries of sequence blockIdx.z, wave = head.
+    // DECODE:  one wave per workgroup; rows = 16 heads of token blockIdx.x,
+    //          the token's visible keys split over blockIdx.z.
+    constexpr int NTH = DECODE ? 64 : 256;
+    const int seq = DECODE ? seq_idx[blockIdx.x] : (int)blockIdx.z;
+    const int s0 = DECODE ? (int)blockIdx.x : cu[seq];
+    const int QL = DECODE ? 1 : cu[seq + 1] - s0;
+    const int q0 = DECODE ? 0 : blockIdx.x * 16;
     if (q0 >= QL) return;
     const int tid = threadIdx.x, lane = tid % WAVE, wid = tid / WAVE;
     const int lg = lane >> 4, li = lane & 15;
-    const int h = blockIdx.y * 4 + wid;
+    // head of this lane's A row (li) / of the wave
+    const int h = DECODE ? blockIdx.y * 16 + li : blockIdx.y * 4 + wid;
     const bool head_ok = h < H;
     const int Dk = C + R;
     const int hist = positions[s0];
@@ -196,7 +204,7 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
 
     bf16x8 a_q[KSTEPS];
     {
-        const int row = q0 + li;
+        const int row = DECODE ? 0 : q0 + li;
         const bool ok = head_ok && row < QL;
         const unsigned short* qa = q_abs + ((long)h * Tn + s0 + row) * C;
         const unsigned short* qr = q_rot + (long)(s0 + row) * qr_tok +
@@ -223,13 +231,19 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
     for (int nb = 0; nb < KSTEPS * 2; ++nb) o_acc[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     const int last_row = min(q0 + 15, QL - 1);
-    const int kv_lo = max(0, hist + q0 - window + 1);
-    const int kv_end = hist + last_row + 1;
+    int kv_lo = max(0, hist + q0 - window + 1);
+    int kv_end = hist + last_row + 1;
+    if (DECODE && gridDim.z > 1) {
+        int per = (kv_end - kv_lo + (int)gridDim.z - 1) / (int)gridDim.z;
+        per = (per + LM_TN - 1) / LM_TN * LM_TN;
+        kv_lo += blockIdx.z * per;
+        kv_end = min(kv_end, kv_lo + per);
+    }
 
     for (int kb = kv_lo; kb < kv_end; kb += LM_TN) {
         __syncthreads();   // previous tile's reads of k_s are done
         constexpr int UNITS = DKP / 8;
-        for (int i = tid; i < LM_TN * UNITS; i += 256) {
+        for (int i = tid; i < LM_TN * UNITS; i += NTH) {
             const int key = i / UNITS, d = (i - key * UNITS) * 8;
             const int gk = kb + key;
             short8 raw = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -260,9 +274,12 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
         for (int f = 0; f < LM_TN / 16; ++f) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int qrow = q0 + lg * 4 + r;
-                const int back = hist + qrow - (kb + f * 16 + li);
-                const bool vis = qrow < QL && back >= 0 && back < window;
+                // DECODE: every row is the same token (rows are heads)
+                const int qrow = DECODE ? 0 : q0 + lg * 4 + r;
+                const int key = kb + f * 16 + li;
+                const int back = hist + qrow - key;
+                const bool vis = qrow < QL && back >= 0 && back < window &&
+                                 key < kv_end;
                 sfrag[f][r] = vis ? sfrag[f][r] * scale : -1e30f;
                 pmax[r] = fmaxf(pmax[r], sfrag[f][r]);
             }
@@ -322,6 +339,37 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
                     a_lo, bv, o_acc[nb], 0, 0, 0);
             }
         }
+    }
+    if (DECODE) {
+        // C layout: this lane holds heads (rows) lg*4 + r, column li
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int hh = blockIdx.y * 16 + lg * 4 + r;
+            if (hh >= H) continue;
+            if (gridDim.z > 1) {
+                const long row = ((long)blockIdx.z * H + hh) * Tn + s0;
+#pragma unroll
+                for (int nb = 0; nb < KSTEPS * 2; ++nb) {
+                    const int c = nb * 16 + li;
+                    if (c < C) part_acc[row * C + c] = o_acc[nb][r];
+                }
+                if (li == 0) {
+                    part_ml[row * 2] = m_run[r];
+                    part_ml[row * 2 + 1] = l_run[r];
+                }
+            } else {
+                const float g = 1.f / (1.f + expf(-bf2f(
+                    gate[(long)s0 * gate_tok + hh])));
+                const float inv = l_run[r] > 0.f ? g / l_run[r] : 0.f;
+                unsigned short* orow = out + ((long)hh * Tn + s0) * C;
+#pragma unroll
+                for (int nb = 0; nb < KSTEPS * 2; ++nb) {
+                    const int c = nb * 16 + li;
+                    if (c < C) orow[c] = f2bf(o_acc[nb][r] * inv);
+                }
+            }
+        }
+        return;
     }
     if (!head_ok) return;
 #pragma unroll
@@ -527,31 +575,51 @@ extern "C" int launch_latent_attn(const void* q_abs, const void* q_rot,
         C, R, bs, window, scale, s);
 }
 
-#define LM_CASE(N)                                                            \
-    latent_attn_mfma_kernel<N><<<grid, 256, 0, s>>>(                          \
+#define LM_CASE(N, DEC, TH)                                                   \
+    latent_attn_mfma_kernel<N, DEC><<<grid, TH, 0, s>>>(                      \
         (const unsigned short*)q_abs, (const unsigned short*)q_rot, qr_tok,   \
         qr_head, (const unsigned short*)gate, gate_tok,                       \
         (const unsigned short*)cache, block_table, bt_stride, cu, positions,  \
-        (unsigned short*)out, Tn, H, C, R, bs, window, scale)
+        seq_idx, (unsigned short*)out, part_acc, part_ml, Tn, H, C, R, bs,    \
+        window, scale)
 
-// bf16 prompt portions on the matrix cores. Returns nonzero when the shape
-// is not covered (row width not a multiple of 8 or above 576) and the
-// caller should use the generic kernel.
+// bf16 on the matrix cores: prompt portions (max_qlen >= 16; 16-query x
+// 4-head workgroups over B sequences) or pure decode steps (max_qlen == 1;
+// one wave per token x 16 heads x key split, merged by the combine kernel
+// when splits > 1). Returns nonzero when the shape is not covered (row
+// width not a multiple of 8 or above 576): the caller then uses the
+// generic kernel.
 extern "C" int launch_latent_attn_mfma(
     const void* q_abs, const void* q_rot, long qr_tok, long qr_head,
     const void* gate, long gate_tok, const void* cache,
     const int* block_table, int bt_stride, const int* cu,
-    const int* positions, void* out, int Tn, int B, int max_qlen, int H,
-    int C, int R, int bs, int window, float scale, hipStream_t s) {
+    const int* positions, const int* seq_idx, void* out, float* part_acc,
+    float* part_ml, int splits, int Tn, int B, int max_qlen, int H, int C,
+    int R, int bs, int window, float scale, hipStream_t s) {
     const int Dk = C + R;
     if (Dk % 8 != 0 || Dk > 576) return 1;
     if (Tn == 0 || B == 0) return 0;
-    const dim3 grid((max_qlen + 15) / 16, (H + 3) / 4, B);
     const int ksteps = (Dk + 31) / 32;
-    if (ksteps <= 4) LM_CASE(4);
-    else if (ksteps <= 8) LM_CASE(8);
-    else if (ksteps <= 12) LM_CASE(12);
-    else LM_CASE(18);
+    if (max_qlen == 1) {
+        const dim3 grid(Tn, (H + 15) / 16, splits);
+        if (ksteps <= 4) LM_CASE(4, true, 64);
+        else if (ksteps <= 8) LM_CASE(8, true, 64);
+        else if (ksteps <= 12) LM_CASE(12, true, 64);
+        else LM_CASE(18, true, 64);
+        if (splits > 1) {
+            const dim3 g2(Tn, (H + LA_WAVES - 1) / LA_WAVES);
+            latent_attn_combine_kernel<unsigned short>
+                <<<g2, LA_WAVES * WAVE, 0, s>>>(
+                    part_acc, part_ml, (const unsigned short*)gate, gate_tok,
+                    (unsigned short*)out, splits, Tn, H, C);
+        }
+        return 0;
+    }
+    const dim3 grid((max_qlen + 15) / 16, (H + 3) / 4, B);
+    if (ksteps <= 4) LM_CASE(4, false, 256);
+    else if (ksteps <= 8) LM_CASE(8, false, 256);
+    else if (ksteps <= 12) LM_CASE(12, false, 256);
+    else LM_CASE(18, false, 256);
     return 0;
 }
 

@@ -166,3 +166,25 @@ def test_lightning_chunks_and_state(dtype, H, D, Dv):
     torch.testing.assert_close(o1 / scale, o2 / scale, rtol=1e-4, atol=2e-5)
     torch.testing.assert_close(s1, s2, rtol=1e-4, atol=1e-4 * float(
         s2.abs().max()))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,C,R,window", [(3, 20, 4, 7), (8, 96, 16, 40),
+                                          (16, 512, 64, 300), (20, 130, 24, 90)])
+def test_latent_attention_decode_step(dtype, H, C, R, window):
+    """A step of single tokens (one row per sequence) at scattered
+    positions: the key-split decode kernels and their merge."""
+    torch.manual_seed(5)
+    bs = 16
+    lens, starts = [1, 1, 1, 1, 1], [0, 47, 15, 200, 95]
+    m = batch_meta(lens, starts, bs, 32)
+    T = m["T"]
+    cache = torch.randn(32, bs, C + R, device=DEV).to(dtype)
+    q_abs = (torch.randn(H, T, C, device=DEV) * C ** -0.5).to(dtype)
+    q_rot = torch.randn(T, H, R, device=DEV).to(dtype)
+    gate = torch.randn(T, H, device=DEV).to(dtype)
+    o1 = ops.latent_attn(q_abs, q_rot, gate, cache, m["bt"], m["pos"],
+                         m["seq"], m["cu"], window, 0.3, 1)
+    o2 = ref.latent_attn(q_abs, q_rot, gate, cache, m["bt"], m["pos"],
+                         m["seq"], m["cu"], window, 0.3)
+    torch.testing.assert_close(o1.float(), o2.float(), **tol(dtype))
