@@ -163,7 +163,7 @@ constexpr int LM_TN = 32;
 constexpr int LM_PAD = 8;
 
 template <int KSTEPS, bool DECODE>
-__global__ void __launch_bounds__(DECODE ? 64 : 256)
+__global__ void __launch_bounds__(256)
 latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
                         const unsigned short* __restrict__ q_rot, long qr_tok,
                         long qr_head, const unsigned short* __restrict__ gate,
@@ -185,9 +185,12 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
     __shared__ __attribute__((aligned(16))) unsigned short p_lo[64 * PS];
 
     // PREFILL: rows = 16 queries of sequence blockIdx.z, wave = head.
-    // DECODE:  one wave per workgroup; rows = 16 heads of token blockIdx.x,
-    //          the token's visible keys split over blockIdx.z.
-    constexpr int NTH = DECODE ? 64 : 256;
+    // DECODE:  rows = 16 heads of token blockIdx.x, the token's visible keys
+    //          split over blockIdx.z. The four waves stage the key tile
+    //          together, each recomputes the (small) score tile, and each
+    //          accumulates every fourth 16-column block of the output.
+    constexpr int NTH = 256;
+    constexpr int NBW = DECODE ? (KSTEPS * 2 + 3) / 4 : KSTEPS * 2;
     const int seq = DECODE ? seq_idx[blockIdx.x] : (int)blockIdx.z;
     const int s0 = DECODE ? (int)blockIdx.x : cu[seq];
     const int QL = DECODE ? 1 : cu[seq + 1] - s0;
@@ -211,24 +214,26 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
                                    (long)h * qr_head;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
-            short8 raw;
+            const int c0 = ks * 32 + lg * 8;
+            short8 raw = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (ok && c0 + 8 <= C) {
+                // C is a multiple of 8 here: the unit lies inside the
+                // (16 B aligned) absorbed-query row
+                raw = *reinterpret_cast<const short8*>(qa + c0);
+            } else if (ok && c0 < Dk) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int c = ks * 32 + lg * 8 + e;
-                unsigned short v = 0;
-                if (ok && c < C) v = qa[c];
-                else if (ok && c < Dk) v = qr[c - C];
-                raw[e] = (short)v;
+                for (int e = 0; e < 8; ++e)
+                    raw[e] = (short)qr[c0 + e - C];
             }
             a_q[ks] = __builtin_bit_cast(bf16x8, raw);
         }
     }
     float m_run[4], l_run[4];
-    f32x4 o_acc[KSTEPS * 2];
+    f32x4 o_acc[NBW];
 #pragma unroll
     for (int r = 0; r < 4; ++r) { m_run[r] = -1e30f; l_run[r] = 0.f; }
 #pragma unroll
-    for (int nb = 0; nb < KSTEPS * 2; ++nb) o_acc[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < NBW; ++j) o_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     const int last_row = min(q0 + 15, QL - 1);
     int kv_lo = max(0, hist + q0 - window + 1);
@@ -317,26 +322,27 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
 #pragma unroll
         for (int r = 0; r < 4; ++r) l_run[r] = l_run[r] * alpha[r] + psum[r];
 #pragma unroll
-        for (int nb = 0; nb < KSTEPS * 2; ++nb)
+        for (int j = 0; j < NBW; ++j)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) o_acc[nb][r] *= alpha[r];
+            for (int r = 0; r < 4; ++r) o_acc[j][r] *= alpha[r];
         __syncthreads();   // weight tile visible to the wave's other lanes
         const bf16x8 a_hi = *reinterpret_cast<const bf16x8*>(
             p_hi + (wid * 16 + li) * PS + lg * 8);
         const bf16x8 a_lo = *reinterpret_cast<const bf16x8*>(
             p_lo + (wid * 16 + li) * PS + lg * 8);
 #pragma unroll
-        for (int nb = 0; nb < KSTEPS * 2; ++nb) {
+        for (int j = 0; j < NBW; ++j) {
+            const int nb = DECODE ? j * 4 + wid : j;
             if (nb * 16 < C) {
                 short8 raw;
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
                     raw[e] = (short)k_s[(lg * 8 + e) * KS + nb * 16 + li];
                 const bf16x8 bv = __builtin_bit_cast(bf16x8, raw);
-                o_acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                    a_hi, bv, o_acc[nb], 0, 0, 0);
-                o_acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                    a_lo, bv, o_acc[nb], 0, 0, 0);
+                o_acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    a_hi, bv, o_acc[j], 0, 0, 0);
+                o_acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    a_lo, bv, o_acc[j], 0, 0, 0);
             }
         }
     }
@@ -349,11 +355,11 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
             if (gridDim.z > 1) {
                 const long row = ((long)blockIdx.z * H + hh) * Tn + s0;
 #pragma unroll
-                for (int nb = 0; nb < KSTEPS * 2; ++nb) {
-                    const int c = nb * 16 + li;
-                    if (c < C) part_acc[row * C + c] = o_acc[nb][r];
+                for (int j = 0; j < NBW; ++j) {
+                    const int c = (j * 4 + wid) * 16 + li;
+                    if (c < C) part_acc[row * C + c] = o_acc[j][r];
                 }
-                if (li == 0) {
+                if (li == 0 && wid == 0) {
                     part_ml[row * 2] = m_run[r];
                     part_ml[row * 2 + 1] = l_run[r];
                 }
@@ -363,9 +369,9 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
                 const float inv = l_run[r] > 0.f ? g / l_run[r] : 0.f;
                 unsigned short* orow = out + ((long)hh * Tn + s0) * C;
 #pragma unroll
-                for (int nb = 0; nb < KSTEPS * 2; ++nb) {
-                    const int c = nb * 16 + li;
-                    if (c < C) orow[c] = f2bf(o_acc[nb][r] * inv);
+                for (int j = 0; j < NBW; ++j) {
+                    const int c = (j * 4 + wid) * 16 + li;
+                    if (c < C) orow[c] = f2bf(o_acc[j][r] * inv);
                 }
             }
         }
@@ -381,9 +387,9 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
         const float inv = l_run[r] > 0.f ? g / l_run[r] : 0.f;
         unsigned short* orow = out + ((long)h * Tn + s0 + qrow) * C;
 #pragma unroll
-        for (int nb = 0; nb < KSTEPS * 2; ++nb) {
-            const int c = nb * 16 + li;
-            if (c < C) orow[c] = f2bf(o_acc[nb][r] * inv);
+        for (int j = 0; j < NBW; ++j) {
+            const int c = j * 16 + li;
+            if (c < C) orow[c] = f2bf(o_acc[j][r] * inv);
         }
     }
 }
@@ -586,9 +592,9 @@ extern "C" int launch_latent_attn(const void* q_abs, const void* q_rot,
 // bf16 on the matrix cores: prompt portions (max_qlen >= 16; 16-query x
 // 4-head workgroups over B sequences) or pure decode steps (max_qlen == 1;
 // one wave per token x 16 heads x key split, merged by the combine kernel
-// when splits > 1). Returns nonzero when the shape is not covered (row
-// width not a multiple of 8 or above 576): the caller then uses the
-// generic kernel.
+// when splits > 1). Returns nonzero when the shape is not covered (latent
+// or rotated width not a multiple of 8, or their sum above 576): the caller
+// then uses the generic kernel.
 extern "C" int launch_latent_attn_mfma(
     const void* q_abs, const void* q_rot, long qr_tok, long qr_head,
     const void* gate, long gate_tok, const void* cache,
@@ -597,15 +603,15 @@ extern "C" int launch_latent_attn_mfma(
     float* part_ml, int splits, int Tn, int B, int max_qlen, int H, int C,
     int R, int bs, int window, float scale, hipStream_t s) {
     const int Dk = C + R;
-    if (Dk % 8 != 0 || Dk > 576) return 1;
+    if (C % 8 != 0 || R % 8 != 0 || Dk > 576) return 1;
     if (Tn == 0 || B == 0) return 0;
     const int ksteps = (Dk + 31) / 32;
     if (max_qlen == 1) {
         const dim3 grid(Tn, (H + 15) / 16, splits);
-        if (ksteps <= 4) LM_CASE(4, true, 64);
-        else if (ksteps <= 8) LM_CASE(8, true, 64);
-        else if (ksteps <= 12) LM_CASE(12, true, 64);
-        else LM_CASE(18, true, 64);
+        if (ksteps <= 4) LM_CASE(4, true, 256);
+        else if (ksteps <= 8) LM_CASE(8, true, 256);
+        else if (ksteps <= 12) LM_CASE(12, true, 256);
+        else LM_CASE(18, true, 256);
         if (splits > 1) {
             const dim3 g2(Tn, (H + LA_WAVES - 1) / LA_WAVES);
             latent_attn_combine_kernel<unsigned short>
