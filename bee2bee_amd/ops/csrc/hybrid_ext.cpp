@@ -247,13 +247,14 @@ Tensor latent_attn(const Tensor& q_abs, const Tensor& q_rot,
         pm = part_ml.data_ptr<float>();
     };
     // bf16 prompt portions (16-query tiles) and pure decode steps (16-head
-    // tiles, keys split until ~1024 workgroups) run on the matrix cores;
+    // tiles, keys split until ~768 workgroups) run on the matrix cores;
     // fp32, short mixed steps and uncovered shapes take the generic kernel
     if (c == 0 && (max_qlen >= 16 || max_qlen == 1) && C % 8 == 0 &&
         R % 8 == 0 && C + R <= 576) {
         long sp = 1;
         if (max_qlen == 1) {
-            sp = 1024 / std::max<long>(1, (long)Tn * ((H + 15) / 16));
+            // one resident round: 3 workgroups fit a CU's LDS, 256 CUs
+            sp = 768 / std::max<long>(1, (long)Tn * ((H + 15) / 16));
             sp = std::max<long>(1, std::min<long>({sp, 16, (window + 63) / 64}));
             if (sp > 1) alloc_parts(sp);
         }

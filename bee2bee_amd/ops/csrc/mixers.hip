@@ -394,37 +394,40 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
     }
 }
 
-// merge the key-split partials of one (token, head): wave per row
+// merge the key-split partials of one (token, head): one wave per row.
+// Lane z < splits holds share z's (max, sum); the merge weights
+// exp(m_z - M) are computed once and broadcast by shuffle.
 template <typename T>
-__global__ void __launch_bounds__(LA_WAVES * WAVE)
+__global__ void __launch_bounds__(WAVE)
 latent_attn_combine_kernel(const float* __restrict__ part_acc,
                            const float* __restrict__ part_ml,
                            const T* __restrict__ gate, long gate_tok,
                            T* __restrict__ out, int splits, int Tn, int H,
                            int C) {
-    const int t = blockIdx.x;
-    const int lane = threadIdx.x % WAVE;
-    const int h = blockIdx.y * LA_WAVES + threadIdx.x / WAVE;
-    if (h >= H) return;
-    float M = -INFINITY;
-    for (int z = 0; z < splits; ++z)
-        M = fmaxf(M, part_ml[(((long)z * H + h) * Tn + t) * 2]);
-    float L = 0.f;
-    for (int z = 0; z < splits; ++z) {
-        const long row = ((long)z * H + h) * Tn + t;
-        const float l = part_ml[row * 2 + 1];
-        if (l > 0.f) L += l * expf(part_ml[row * 2] - M);
+    const int t = blockIdx.x, h = blockIdx.y;
+    const int lane = threadIdx.x;
+    float m = -INFINITY, l = 0.f;
+    if (lane < splits) {
+        const long row = ((long)lane * H + h) * Tn + t;
+        m = part_ml[row * 2];
+        l = part_ml[row * 2 + 1];
     }
+    const float M = wave_max(l > 0.f ? m : -INFINITY);
+    const float w = l > 0.f ? expf(m - M) : 0.f;
+    const float L = wave_sum(l * w);
     const float g = 1.f / (1.f + expf(-ldf(gate + (long)t * gate_tok + h)));
+    const float r = g / L;
     T* o = out + ((long)h * Tn + t) * C;
-    for (int c = lane; c < C; c += WAVE) {
+    // uniform trip count: every lane takes part in every shuffle
+    for (int c0 = 0; c0 < C; c0 += WAVE) {
+        const int c = c0 + lane;
         float a = 0.f;
         for (int z = 0; z < splits; ++z) {
-            const long row = ((long)z * H + h) * Tn + t;
-            if (part_ml[row * 2 + 1] > 0.f)
-                a += part_acc[row * C + c] * expf(part_ml[row * 2] - M);
+            const float wz = __shfl(w, z);
+            if (c < C)
+                a += part_acc[(((long)z * H + h) * Tn + t) * C + c] * wz;
         }
-        stf(o + c, a * g / L);
+        if (c < C) stf(o + c, a * r);
     }
 }
 
@@ -551,8 +554,8 @@ static int latent_attn_dispatch(const void* q_abs, const void* q_rot,
         LA_CASE(12) LA_CASE(16)
     }
     if (splits > 1) {
-        const dim3 g2(Tn, (H + LA_WAVES - 1) / LA_WAVES);
-        latent_attn_combine_kernel<TT><<<g2, LA_WAVES * WAVE, 0, s>>>(
+        const dim3 g2(Tn, H);
+        latent_attn_combine_kernel<TT><<<g2, WAVE, 0, s>>>(
             part_acc, part_ml, (const TT*)gate, gate_tok, (TT*)out, splits,
             Tn, H, C);
     }
@@ -613,9 +616,9 @@ extern "C" int launch_latent_attn_mfma(
         else if (ksteps <= 12) LM_CASE(12, true, 256);
         else LM_CASE(18, true, 256);
         if (splits > 1) {
-            const dim3 g2(Tn, (H + LA_WAVES - 1) / LA_WAVES);
+            const dim3 g2(Tn, H);
             latent_attn_combine_kernel<unsigned short>
-                <<<g2, LA_WAVES * WAVE, 0, s>>>(
+                <<<g2, WAVE, 0, s>>>(
                     part_acc, part_ml, (const unsigned short*)gate, gate_tok,
                     (unsigned short*)out, splits, Tn, H, C);
         }
