@@ -318,6 +318,21 @@ def seed_model(name, path, port):
     asyncio.run(_run())
 
 
+@cli.command("trace-run", context_settings={"ignore_unknown_options": True})
+@click.argument("args", nargs=-1, type=click.UNPROCESSED)
+def trace_run_cmd(args):
+    """Replay a token trace through a served model and write the logits at
+    the wanted places (same options as bin/trace_run: --model DIR --dtype
+    bfloat16|float32 --out DIR --max-tokens N; steps on standard input)."""
+    import sys
+
+    from .engine.trace import main as trace_main
+    from .ops.build import ensure_built
+
+    ensure_built()
+    sys.exit(trace_main(list(args)))
+
+
 @cli.command("bench")
 @click.option("--model", default="llama3-8b")
 @click.option("--batch", default=64, type=int)
