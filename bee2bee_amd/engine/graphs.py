@@ -51,7 +51,8 @@ class DecodeGraphs:
         # state, so it must never touch a live sequence's slot
         self.state_slots = (
             torch.zeros(max_batch, dtype=torch.int32, device=dev)
-            if runner.spec.is_hybrid else None)
+            if getattr(getattr(runner, "spec", None), "is_hybrid", False)
+            else None)
         self.scratch = None  # (block_table row tensor, state slot int)
         self.logits: Dict[int, torch.Tensor] = {}
         self._graphs: Dict[int, torch.cuda.CUDAGraph] = {}

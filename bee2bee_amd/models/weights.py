@@ -580,6 +580,94 @@ def _save_gpt2(weights: "ModelWeights", out_dir: str, tensors, cpu) -> None:
         json.dump(cfg, f, indent=1)
 
 
+def nukopel_config(spec: ModelSpec) -> Dict:
+    """The config.json dict of a hybrid spec (inverse of nukopel_spec)."""
+    layers = []
+    for l in spec.layer_specs:
+        m, f = l.mixer, l.ffn
+        if m.kind == "latent_attention":
+            mixer = {"heads": m.heads, "dim": m.dim, "rot_dim": m.rot_dim,
+                     "vdim": m.vdim, "kv_rank": m.kv_rank,
+                     "mask": {"size": m.window},
+                     "rot": {"base": m.rope_base, "dims": m.rope_dims},
+                     "scale": m.scale}
+        else:
+            mixer = {"heads": m.heads, "dim": m.dim, "vdim": m.vdim,
+                     "decay": list(m.decay)}
+        mlp = None
+        if f is not None:
+            mlp = {"kind": "moe",
+                   "expert": {"ff": f.ff, "limit": f.limit},
+                   "router": {"experts": f.n_experts, "top": f.top_k},
+                   "shared": ({"ff": f.shared_ff, "limit": f.shared_limit}
+                              if f.shared_ff else None)}
+        layers.append({"type": m.kind, "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Nukopel", "vocab": spec.vocab_size,
+            "width": spec.hidden_size, "canon": {"taps": spec.canon_taps},
+            "embedding": {"scale": spec.embed_scale},
+            "norm": {"eps": spec.rms_eps}, "max_seq_len": spec.max_seq_len,
+            "layers": layers}
+
+
+def _save_nukopel(weights: "ModelWeights", out_dir: str, tensors, cpu) -> None:
+    """Nukopel-format shard + config: the fused/stacked engine layout split
+    back into the checkpoint's tensors (bf16, [out, in])."""
+    from safetensors.torch import save_file
+
+    s = weights.spec
+
+    def put(name: str, t: torch.Tensor) -> None:
+        tensors[name] = cpu(t).to(torch.bfloat16).contiguous()
+
+    def gain(name: str, g: float) -> None:
+        tensors[name] = torch.tensor(g, dtype=torch.bfloat16)
+
+    put("embed", weights.embed)
+    put("head", weights.lm_head)
+    gain("final.norm", weights.final_gain)
+    for i, l in enumerate(s.layer_specs):
+        lw, p, m, f = weights.layers[i], f"l{i}.", l.mixer, l.ffn
+        names = ("norm1", "norm1b") + (("norm2", "norm2b") if f else ())
+        for n, g in zip(names, lw.gains):
+            gain(p + n, g)
+        if lw.canon is not None:
+            put(p + "canon1", lw.canon)
+        H = m.heads
+        if m.kind == "latent_attention":
+            q, dkv, g = torch.split(
+                lw.wqkv, [m.q_size, m.cache_dim, H], dim=0)
+            put(p + "mix.q", q)
+            put(p + "mix.dkv", dkv)
+            put(p + "mix.g", g)
+            put(p + "mix.dkv.norm", lw.kv_norm)
+            put(p + "mix.uk", lw.w_uk.reshape(H * m.dim, m.kv_rank))
+            put(p + "mix.uv", lw.w_uv.transpose(1, 2).reshape(
+                H * m.vdim, m.kv_rank))
+        else:
+            q, k, v, g = torch.split(
+                lw.wqkv, [H * m.dim, H * m.dim, H * m.vdim, H * m.vdim], dim=0)
+            for n, t in (("q", q), ("k", k), ("v", v), ("g", g)):
+                put(p + "mix." + n, t)
+            put(p + "mix.norm", lw.out_norm)
+        put(p + "mix.o", lw.wo)
+        if f is None:
+            continue
+        put(p + "mlp.router", lw.moe_gate)
+        for e in range(f.n_experts):
+            ge, up = torch.split(lw.moe_w_gate_up[e], [f.ff, f.ff], dim=0)
+            put(f"{p}mlp.e{e}.gate", ge)
+            put(f"{p}mlp.e{e}.up", up)
+            put(f"{p}mlp.e{e}.down", lw.moe_w_down[e])
+        if f.shared_ff:
+            ge, up = torch.split(lw.w_gate_up, [f.shared_ff, f.shared_ff], dim=0)
+            put(p + "mlp.shared.gate", ge)
+            put(p + "mlp.shared.up", up)
+            put(p + "mlp.shared.down", lw.w_down)
+    save_file(tensors, os.path.join(out_dir, "model.safetensors"))
+    with open(os.path.join(out_dir, "config.json"), "w") as fh:
+        json.dump(nukopel_config(s), fh, indent=1)
+
+
 def iter_safetensors(model_path: str) -> Iterator[Tuple[str, torch.Tensor]]:
     """Yield (name, tensor) from every *.safetensors shard in a directory."""
     from safetensors import safe_open
@@ -607,6 +695,9 @@ def save_hf(weights: ModelWeights, out_dir: str) -> None:
 
     if s.arch == "gpt2":
         _save_gpt2(weights, out_dir, tensors, cpu)
+        return
+    if s.is_hybrid:
+        _save_nukopel(weights, out_dir, tensors, cpu)
         return
 
     if weights.embed is not None:

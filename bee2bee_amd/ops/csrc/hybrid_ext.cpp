@@ -38,9 +38,11 @@ int launch_latent_attn_mfma(const void*, const void*, long, long, const void*,
                             const int*, const int*, void*, float*, float*,
                             int, int, int, int, int, int, int, int, int,
                             float, hipStream_t);
+int lightning_segment_tokens();
 int launch_lightning(const void*, const void*, const void*, long,
                      const float*, float*, const int*, const int*, const int*,
-                     float*, int, int, int, int, int, hipStream_t);
+                     float*, float*, int, int, int, int, int, int,
+                     hipStream_t);
 }
 
 namespace {
@@ -313,14 +315,26 @@ Tensor lightning_attn(const Tensor& q, const Tensor& k, const Tensor& v,
                 state.size(2) == D && state.size(3) == Dv);
     const int B = (int)cu.numel() - 1;
     TORCH_CHECK(state_slots.numel() == B && positions.numel() == T);
-    Tensor out = torch::empty({T, (long)H * Dv},
-                              q.options().dtype(torch::kFloat32));
+    auto f32opt = q.options().dtype(torch::kFloat32);
+    Tensor out = torch::empty({T, (long)H * Dv}, f32opt);
+    // chunks longer than one segment: segments run in parallel from zero
+    // states and a scan carries the true state across them. n_seg bounds
+    // the batch's segment count without reading the lengths.
+    const long seg = lightning_segment_tokens();
+    long n_seg = 0;
+    Tensor ws;
+    float* wsp = nullptr;
+    if (max_qlen > seg) {
+        n_seg = T / seg + B;
+        ws = torch::empty({n_seg, (long)H, (long)D, (long)Dv}, f32opt);
+        wsp = ws.data_ptr<float>();
+    }
     const int rc = launch_lightning(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0),
         decay.data_ptr<float>(), state.data_ptr<float>(),
         state_slots.data_ptr<int>(), cu.data_ptr<int>(),
-        positions.data_ptr<int>(), out.data_ptr<float>(), B, H, D, Dv, c,
-        stream());
+        positions.data_ptr<int>(), out.data_ptr<float>(), wsp, (int)n_seg, B,
+        H, D, Dv, c, stream());
     TORCH_CHECK(rc == 0, "lightning_attn: key dim must be <= 256");
     return out;
 }

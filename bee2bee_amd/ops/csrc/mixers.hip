@@ -443,7 +443,38 @@ DEV_INLINE float silu_f(float x) { return x / (1.f + expf(-x)); }
 // round of LI_TB tokens the block stages silu(q), silu(k) (all D rows) and
 // silu(v) (its columns) in LDS once — wave g then reads q/k as broadcasts —
 // and the four row groups' partial outputs are summed through LDS.
-template <typename T, int DPT>
+//
+// MODE 0: a whole chunk per workgroup, from the sequence's carried state.
+// Long chunks are cut into LI_SEG-token segments that run in parallel:
+// MODE 1: a segment from a ZERO state; local outputs to `out`, the
+//         segment's final local state to the workspace `ws`;
+//   (lightning_scan_kernel then turns ws into the true state at each
+//    segment's start and writes the sequence's final state to its slot)
+// MODE 2: adds lam^(i+1) * S_start^T q_i to the segment's outputs (state
+//         fixed, no update), i = token index within the segment.
+// S_t = lam^(i+1) S_start + S_local,t, so modes 1+2 equal mode 0 up to fp32
+// summation order.
+constexpr int LI_SEG = 256;
+
+// segment index -> (sequence, first row, end row); false when out of range
+DEV_INLINE bool li_segment(const int* __restrict__ cu, int B, int seg,
+                           int* b_out, int* lo, int* hi) {
+    int first = 0;
+    for (int b = 0; b < B; ++b) {
+        const int len = cu[b + 1] - cu[b];
+        const int n = (len + LI_SEG - 1) / LI_SEG;
+        if (seg < first + n) {
+            *b_out = b;
+            *lo = cu[b] + (seg - first) * LI_SEG;
+            *hi = min(cu[b + 1], *lo + LI_SEG);
+            return true;
+        }
+        first += n;
+    }
+    return false;
+}
+
+template <typename T, int DPT, int MODE>
 __global__ void __launch_bounds__(LI_COLS * LI_GROUPS)
 lightning_kernel(const T* __restrict__ q, const T* __restrict__ k,
                  const T* __restrict__ v, long tok_stride,
@@ -453,14 +484,22 @@ lightning_kernel(const T* __restrict__ q, const T* __restrict__ k,
                  const int* __restrict__ cu,
                  const int* __restrict__ positions,
                  float* __restrict__ out,          // [Tn, H * Dv]
-                 int H, int D, int Dv) {
+                 float* __restrict__ ws,           // [segments, H, D, Dv]
+                 int B, int H, int D, int Dv) {
     constexpr int DMAX = DPT * LI_GROUPS;
     __shared__ float qs[LI_TB][DMAX];
     __shared__ float ks[LI_TB][DMAX];
     __shared__ float vs[LI_TB][LI_COLS];
     __shared__ float red[LI_TB][LI_GROUPS][LI_COLS];
-    const int b = blockIdx.x, h = blockIdx.y;
-    const int lo = cu[b], hi = cu[b + 1];
+    const int h = blockIdx.y;
+    int b, lo, hi;
+    if (MODE == 0) {
+        b = blockIdx.x;
+        lo = cu[b];
+        hi = cu[b + 1];
+    } else if (!li_segment(cu, B, blockIdx.x, &b, &lo, &hi)) {
+        return;
+    }
     if (hi <= lo) return;
     const int nth = LI_COLS * LI_GROUPS;
     const int g = threadIdx.x / LI_COLS, col = threadIdx.x % LI_COLS;
@@ -469,8 +508,11 @@ lightning_kernel(const T* __restrict__ q, const T* __restrict__ k,
     const bool live = dv < Dv;
     const int d0 = g * DPT;
     const float lam = decay[h];
-    float* st = state + (((long)state_slots[b] * H + h) * D) * Dv + dv;
-    const bool fresh = positions[lo] == 0;
+    const float log_lam = logf(lam);
+    float* st = MODE == 0
+        ? state + (((long)state_slots[b] * H + h) * D) * Dv + dv
+        : ws + (((long)blockIdx.x * H + h) * D) * Dv + dv;
+    const bool fresh = MODE == 1 || (MODE == 0 && positions[lo] == 0);
     float s[DPT];
 #pragma unroll
     for (int i = 0; i < DPT; ++i) {
@@ -483,22 +525,30 @@ lightning_kernel(const T* __restrict__ q, const T* __restrict__ k,
             const int tt = idx / DMAX, d = idx - tt * DMAX;
             const long base = (long)(t0 + tt) * tok_stride + (long)h * D + d;
             qs[tt][d] = d < D ? silu_f(ldf(q + base)) : 0.f;
-            ks[tt][d] = d < D ? silu_f(ldf(k + base)) : 0.f;
+            if (MODE != 2) ks[tt][d] = d < D ? silu_f(ldf(k + base)) : 0.f;
         }
-        for (int idx = threadIdx.x; idx < n * LI_COLS; idx += nth) {
-            const int tt = idx / LI_COLS, c = idx - tt * LI_COLS;
-            vs[tt][c] = (c0 + c < Dv)
-                ? silu_f(ldf(v + (long)(t0 + tt) * tok_stride + (long)h * Dv + c0 + c))
-                : 0.f;
+        if (MODE != 2) {
+            for (int idx = threadIdx.x; idx < n * LI_COLS; idx += nth) {
+                const int tt = idx / LI_COLS, c = idx - tt * LI_COLS;
+                vs[tt][c] = (c0 + c < Dv)
+                    ? silu_f(ldf(v + (long)(t0 + tt) * tok_stride +
+                                 (long)h * Dv + c0 + c))
+                    : 0.f;
+            }
         }
         __syncthreads();
         for (int tt = 0; tt < n; ++tt) {
-            const float vv = vs[tt][col];
             float part = 0.f;
+            if (MODE == 2) {
 #pragma unroll
-            for (int i = 0; i < DPT; ++i) {
-                s[i] = lam * s[i] + ks[tt][d0 + i] * vv;
-                part += s[i] * qs[tt][d0 + i];
+                for (int i = 0; i < DPT; ++i) part += s[i] * qs[tt][d0 + i];
+            } else {
+                const float vv = vs[tt][col];
+#pragma unroll
+                for (int i = 0; i < DPT; ++i) {
+                    s[i] = lam * s[i] + ks[tt][d0 + i] * vv;
+                    part += s[i] * qs[tt][d0 + i];
+                }
             }
             red[tt][g][col] = part;
         }
@@ -508,17 +558,56 @@ lightning_kernel(const T* __restrict__ q, const T* __restrict__ k,
             float o = 0.f;
 #pragma unroll
             for (int gg = 0; gg < LI_GROUPS; ++gg) o += red[tt][gg][c];
-            if (c0 + c < Dv)
-                out[(long)(t0 + tt) * H * Dv + (long)h * Dv + c0 + c] = o;
+            if (c0 + c < Dv) {
+                float* op = out + (long)(t0 + tt) * H * Dv + (long)h * Dv +
+                            c0 + c;
+                if (MODE == 2)
+                    *op += o * expf(log_lam * (float)(t0 + tt - lo + 1));
+                else
+                    *op = o;
+            }
         }
     }
-    if (live) {
+    if (MODE != 2 && live) {
 #pragma unroll
         for (int i = 0; i < DPT; ++i) {
             const int d = d0 + i;
             if (d < D) st[(long)d * Dv] = s[i];
         }
     }
+}
+
+// Per (sequence, head), one thread per state element: walk the sequence's
+// segments in order, replacing each segment's local final state in ws by
+// the true state at that segment's start, and leave the sequence's final
+// state in its slot.
+__global__ void lightning_scan_kernel(const float* __restrict__ decay,
+                                      float* __restrict__ state,
+                                      const int* __restrict__ state_slots,
+                                      const int* __restrict__ cu,
+                                      const int* __restrict__ positions,
+                                      float* __restrict__ ws, int H,
+                                      int DDv) {
+    const int b = blockIdx.x, h = blockIdx.y;
+    const int e = blockIdx.z * blockDim.x + threadIdx.x;
+    if (e >= DDv) return;
+    const int lo = cu[b], len = cu[b + 1] - lo;
+    if (len <= 0) return;
+    int first = 0;
+    for (int bb = 0; bb < b; ++bb)
+        first += (cu[bb + 1] - cu[bb] + LI_SEG - 1) / LI_SEG;
+    const float log_lam = logf(decay[h]);
+    float* slot = state + ((long)state_slots[b] * H + h) * DDv + e;
+    float S = positions[lo] == 0 ? 0.f : *slot;
+    const int nseg = (len + LI_SEG - 1) / LI_SEG;
+    for (int sg = 0; sg < nseg; ++sg) {
+        float* w = ws + ((long)(first + sg) * H + h) * DDv + e;
+        const float local = *w;
+        *w = S;
+        const int n = min(LI_SEG, len - sg * LI_SEG);
+        S = expf(log_lam * (float)n) * S + local;
+    }
+    *slot = S;
 }
 
 }  // namespace
@@ -632,43 +721,63 @@ extern "C" int launch_latent_attn_mfma(
     return 0;
 }
 
+#define LI_LAUNCH(N, MODE, GRID)                                              \
+    lightning_kernel<TT, N, MODE><<<GRID, LI_COLS * LI_GROUPS, 0, s>>>(       \
+        (const TT*)q, (const TT*)k, (const TT*)v, tok_stride, decay, state,   \
+        state_slots, cu, positions, out, ws, B, H, D, Dv)
+
 #define LI_CASE(N)                                                            \
     case N:                                                                   \
-        lightning_kernel<TT, N><<<grid, LI_COLS * LI_GROUPS, 0, s>>>(         \
-            (const TT*)q, (const TT*)k, (const TT*)v, tok_stride, decay,      \
-            state, state_slots, cu, positions, out, H, D, Dv);                \
+        if (n_seg == 0) {                                                     \
+            LI_LAUNCH(N, 0, grid);                                            \
+        } else {                                                              \
+            LI_LAUNCH(N, 1, sgrid);                                           \
+            lightning_scan_kernel<<<scan_grid, 256, 0, s>>>(                  \
+                decay, state, state_slots, cu, positions, ws, H, D * Dv);     \
+            LI_LAUNCH(N, 2, sgrid);                                           \
+        }                                                                     \
         break;
 
+// n_seg = 0: one workgroup walks each whole chunk. n_seg > 0 (an upper bound
+// of the number of LI_SEG-token segments in the batch, ws sized for it):
+// segments run in parallel, a scan carries the state across them.
 template <typename TT>
 static int lightning_dispatch(const void* q, const void* k, const void* v,
                               long tok_stride, const float* decay,
                               float* state, const int* state_slots,
                               const int* cu, const int* positions, float* out,
-                              int B, int H, int D, int Dv, hipStream_t s) {
+                              float* ws, int n_seg, int B, int H, int D,
+                              int Dv, hipStream_t s) {
     const int need = (D + LI_GROUPS - 1) / LI_GROUPS;
     const int sizes[] = {2, 8, 16, 32, 64};
     int dpt = 0;
     for (int z : sizes)
         if (z >= need) { dpt = z; break; }
     if (!dpt) return 1;
-    const dim3 grid(B, H, (Dv + LI_COLS - 1) / LI_COLS);
+    const int zc = (Dv + LI_COLS - 1) / LI_COLS;
+    const dim3 grid(B, H, zc), sgrid(n_seg > 0 ? n_seg : 1, H, zc);
+    const dim3 scan_grid(B, H, (D * Dv + 255) / 256);
     switch (dpt) { LI_CASE(2) LI_CASE(8) LI_CASE(16) LI_CASE(32) LI_CASE(64) }
     return 0;
 }
 
 // returns nonzero when the key dim exceeds 256
+extern "C" int lightning_segment_tokens() { return LI_SEG; }
+
 extern "C" int launch_lightning(const void* q, const void* k, const void* v,
                                 long tok_stride, const float* decay,
                                 float* state, const int* state_slots,
                                 const int* cu, const int* positions,
-                                float* out, int B, int H, int D, int Dv,
-                                int f32, hipStream_t s) {
+                                float* out, float* ws, int n_seg, int B,
+                                int H, int D, int Dv, int f32,
+                                hipStream_t s) {
     if (B == 0) return 0;
     if (f32)
         return lightning_dispatch<float>(q, k, v, tok_stride, decay, state,
-                                         state_slots, cu, positions, out, B,
-                                         H, D, Dv, s);
+                                         state_slots, cu, positions, out, ws,
+                                         n_seg, B, H, D, Dv, s);
     return lightning_dispatch<unsigned short>(q, k, v, tok_stride, decay,
                                               state, state_slots, cu,
-                                              positions, out, B, H, D, Dv, s);
+                                              positions, out, ws, n_seg, B, H,
+                                              D, Dv, s);
 }

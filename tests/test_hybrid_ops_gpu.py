@@ -103,7 +103,7 @@ def test_canon_conv_chunks_and_state(dtype, taps):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,C,R,dims,window", [
-    (3, 20, 4, 4, 7), (8, 96, 16, 16, 40), (5, 130, 24, 16, 1),
+    (3, 20, 4, 4, 7), (7, 88, 24, 16, 37), (5, 130, 24, 16, 1),
     (2, 512, 64, 64, 300)])
 def test_latent_store_and_attention(dtype, H, C, R, dims, window):
     torch.manual_seed(3)
@@ -144,12 +144,16 @@ def test_latent_store_and_attention(dtype, H, C, R, dims, window):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,D,Dv", [(2, 8, 12), (4, 32, 32), (3, 128, 80),
+@pytest.mark.parametrize("H,D,Dv", [(2, 8, 12), (4, 48, 64), (3, 128, 80),
                                     (1, 40, 16)])
-def test_lightning_chunks_and_state(dtype, H, D, Dv):
+@pytest.mark.parametrize("lens,starts", [
+    ([70, 1, 2, 5], [0, 9, 0, 130]),
+    # chunks above one segment: the segment-parallel passes and their scan
+    ([600, 1, 300, 257], [0, 9, 130, 0]),
+    ([1, 512], [77, 3])])
+def test_lightning_chunks_and_state(dtype, H, D, Dv, lens, starts):
     torch.manual_seed(4)
-    lens, starts = [70, 1, 2, 5], [0, 9, 0, 130]
-    m = batch_meta(lens, starts, 16, 32)
+    m = batch_meta(lens, starts, 64, 32)
     T = m["T"]
     proj = (torch.randn(T, 2 * H * D + H * Dv + 5, device=DEV)).to(dtype)
     q = proj[:, : H * D].view(T, H, D)
@@ -169,7 +173,7 @@ def test_lightning_chunks_and_state(dtype, H, D, Dv):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,C,R,window", [(3, 20, 4, 7), (8, 96, 16, 40),
+@pytest.mark.parametrize("H,C,R,window", [(3, 20, 4, 7), (6, 72, 8, 50),
                                           (16, 512, 64, 300), (20, 130, 24, 90)])
 def test_latent_attention_decode_step(dtype, H, C, R, window):
     """A step of single tokens (one row per sequence) at scattered

@@ -464,3 +464,28 @@ def test_trace_replay_writes_wanted_logits(tmp_path, monkeypatch, capsys):
     c = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4").reshape(1, -1))
     assert not (out / "1.f32").exists()
     assert rel_err(a, want[[0, 6]]) < 2e-4 and rel_err(c, want[[11]]) < 2e-4
+
+
+def test_checkpoint_roundtrip(tmp_path):
+    """load -> save_hf -> load: the same tensors under the same names, the
+    same config, the same logits."""
+    from safetensors.torch import load_file
+
+    from bee2bee_amd.models.weights import save_hf
+
+    cfg = _cfg("attn-first-no-shared")
+    W = O.random_weights(cfg, seed=18)
+    eng = make_engine(tmp_path, cfg, W)
+    out = tmp_path / "resaved"
+    save_hf(eng.weights, str(out))
+    W2 = load_file(str(out / "model.safetensors"))
+    # the layer without a feed-forward has no second pair of norms
+    assert set(W) - set(W2) == {"l1.norm2", "l1.norm2b"} and set(W2) <= set(W)
+    for k in W2:
+        assert torch.equal(W2[k].float(), W[k].float()), k
+    cfg2 = json.load(open(out / "config.json"))
+    a, b = nukopel_spec("a", cfg), nukopel_spec("b", cfg2)
+    assert a.layer_specs == b.layer_specs
+    assert (a.vocab_size, a.hidden_size, a.canon_taps, a.embed_scale,
+            a.rms_eps) == (b.vocab_size, b.hidden_size, b.canon_taps,
+                           b.embed_scale, b.rms_eps)
