@@ -23,6 +23,36 @@ template <> DEV_INLINE void stf<unsigned short>(unsigned short* p, float v) {
     *p = f2bf(v);
 }
 
+// VEC consecutive elements <-> floats. VEC = 4 moves 16 B (fp32) or 8 B
+// (bf16) per lane and needs rows whose length is a multiple of 4.
+template <typename T, int VEC> DEV_INLINE void ldv(const T* p, float* o);
+template <> DEV_INLINE void ldv<float, 1>(const float* p, float* o) { o[0] = *p; }
+template <> DEV_INLINE void ldv<unsigned short, 1>(const unsigned short* p, float* o) {
+    o[0] = bf2f(*p);
+}
+template <> DEV_INLINE void ldv<float, 4>(const float* p, float* o) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(p);
+    o[0] = v[0]; o[1] = v[1]; o[2] = v[2]; o[3] = v[3];
+}
+template <> DEV_INLINE void ldv<unsigned short, 4>(const unsigned short* p, float* o) {
+    typedef __attribute__((ext_vector_type(4))) unsigned short u16x4;
+    const u16x4 v = *reinterpret_cast<const u16x4*>(p);
+    o[0] = bf2f(v[0]); o[1] = bf2f(v[1]); o[2] = bf2f(v[2]); o[3] = bf2f(v[3]);
+}
+template <typename T, int VEC> DEV_INLINE void stv(T* p, const float* o);
+template <> DEV_INLINE void stv<float, 1>(float* p, const float* o) { *p = o[0]; }
+template <> DEV_INLINE void stv<unsigned short, 1>(unsigned short* p, const float* o) {
+    *p = f2bf(o[0]);
+}
+template <> DEV_INLINE void stv<float, 4>(float* p, const float* o) {
+    *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
+}
+template <> DEV_INLINE void stv<unsigned short, 4>(unsigned short* p, const float* o) {
+    typedef __attribute__((ext_vector_type(4))) unsigned short u16x4;
+    *reinterpret_cast<u16x4*>(p) =
+        u16x4{f2bf(o[0]), f2bf(o[1]), f2bf(o[2]), f2bf(o[3])};
+}
+
 // sum over the block (<= 1024 threads); every thread gets the total
 DEV_INLINE float block_sum(float v, float* red) {
     v = wave_sum(v);
@@ -39,7 +69,7 @@ DEV_INLINE float block_sum(float v, float* red) {
 // ------------------------------------------------------ scalar-gain norms
 // y = x / sqrt(mean(x^2) + eps) * gain; one workgroup per row, the row is
 // held in LDS between the passes.
-template <typename OT>
+template <typename OT, int VEC>
 __global__ void scalar_rmsnorm_kernel(const float* __restrict__ x,
                                       OT* __restrict__ y, int W, float gain,
                                       float eps) {
@@ -49,19 +79,28 @@ __global__ void scalar_rmsnorm_kernel(const float* __restrict__ x,
     const long t = blockIdx.x;
     const float* xr = x + t * (long)W;
     float ss = 0.f;
-    for (int i = threadIdx.x; i < W; i += blockDim.x) {
-        const float v = xr[i];
-        row[i] = v;
-        ss += v * v;
+    for (int i = threadIdx.x * VEC; i < W; i += blockDim.x * VEC) {
+        float v[VEC];
+        ldv<float, VEC>(xr + i, v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            row[i + j] = v[j];
+            ss += v[j] * v[j];
+        }
     }
     const float r = gain / sqrtf(block_sum(ss, red) / (float)W + eps);
     OT* yr = y + t * (long)W;
-    for (int i = threadIdx.x; i < W; i += blockDim.x) stf(yr + i, row[i] * r);
+    for (int i = threadIdx.x * VEC; i < W; i += blockDim.x * VEC) {
+        float v[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = row[i + j] * r;
+        stv<OT, VEC>(yr + i, v);
+    }
 }
 
 // resid += unit(y [+ y2]) * post_gain;  out = unit(resid) * pre_gain
 // (out skipped when HAS_OUT is false). One pass over HBM per operand.
-template <typename YT, typename OT, bool HAS_OUT>
+template <typename YT, typename OT, bool HAS_OUT, int VEC>
 __global__ void add_scalar_rmsnorm_kernel(float* __restrict__ resid,
                                           const YT* __restrict__ y,
                                           const YT* __restrict__ y2,
@@ -75,25 +114,44 @@ __global__ void add_scalar_rmsnorm_kernel(float* __restrict__ resid,
     const YT* yr = y + t * (long)W;
     const YT* y2r = y2 ? y2 + t * (long)W : nullptr;
     float ss = 0.f;
-    for (int i = threadIdx.x; i < W; i += blockDim.x) {
-        float v = ldf(yr + i);
-        if (y2r) v += ldf(y2r + i);
-        row[i] = v;
-        ss += v * v;
+    for (int i = threadIdx.x * VEC; i < W; i += blockDim.x * VEC) {
+        float v[VEC];
+        ldv<YT, VEC>(yr + i, v);
+        if (y2r) {
+            float u[VEC];
+            ldv<YT, VEC>(y2r + i, u);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] += u[j];
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            row[i + j] = v[j];
+            ss += v[j] * v[j];
+        }
     }
     const float ry = post_gain / sqrtf(block_sum(ss, red) / (float)W + eps);
     float* xr = resid + t * (long)W;
     float sx = 0.f;
-    for (int i = threadIdx.x; i < W; i += blockDim.x) {
-        const float v = xr[i] + row[i] * ry;
-        xr[i] = v;
-        row[i] = v;
-        sx += v * v;
+    for (int i = threadIdx.x * VEC; i < W; i += blockDim.x * VEC) {
+        float v[VEC];
+        ldv<float, VEC>(xr + i, v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            v[j] += row[i + j] * ry;
+            row[i + j] = v[j];
+            sx += v[j] * v[j];
+        }
+        stv<float, VEC>(xr + i, v);
     }
     if (!HAS_OUT) return;
     const float rx = pre_gain / sqrtf(block_sum(sx, red) / (float)W + eps);
     OT* orow = out + t * (long)W;
-    for (int i = threadIdx.x; i < W; i += blockDim.x) stf(orow + i, row[i] * rx);
+    for (int i = threadIdx.x * VEC; i < W; i += blockDim.x * VEC) {
+        float v[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = row[i + j] * rx;
+        stv<OT, VEC>(orow + i, v);
+    }
 }
 
 // y = unit(x) * w * sigmoid(gate): x fp32 [T, N], gate raw with row stride
@@ -140,7 +198,7 @@ __global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ y,
 // out[t] = h[t] + sum_d w[c][K-d] * h[t-d], d = 0..K (K = taps-1). Rows
 // before the chunk come from the sequence's state (its last K inputs), rows
 // before position 0 are zero.
-template <typename T>
+template <typename T, int VEC>
 __global__ void canon_conv_kernel(const T* __restrict__ h,
                                   const float* __restrict__ w,   // [C, K+1]
                                   const T* __restrict__ state,   // [S, K, C]
@@ -150,22 +208,29 @@ __global__ void canon_conv_kernel(const T* __restrict__ h,
                                   const int* __restrict__ positions,
                                   T* __restrict__ out, int C, int K) {
     const long t = blockIdx.x;
-    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    const int c = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
     if (c >= C) return;
     const int b = seq_idx[t];
     const int local = (int)t - cu[b];
     const int pos = positions[t];
     const long slot = state_slots[b];
-    const float* wc = w + (long)c * (K + 1);
-    float acc = ldf(h + t * C + c) * (1.f + wc[K]);
+    float acc[VEC], v[VEC];
+    ldv<T, VEC>(h + t * C + c, v);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+        acc[j] = v[j] * (1.f + w[(long)(c + j) * (K + 1) + K]);
     for (int d = 1; d <= K; ++d) {
         if (pos - d < 0) break;
         const int src = local - d;
-        const float v = src >= 0 ? ldf(h + (t - d) * C + c)
-                                 : ldf(state + (slot * K + (K + src)) * C + c);
-        acc += wc[K - d] * v;
+        if (src >= 0)
+            ldv<T, VEC>(h + (t - d) * C + c, v);
+        else
+            ldv<T, VEC>(state + (slot * K + (K + src)) * C + c, v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+            acc[j] += w[(long)(c + j) * (K + 1) + K - d] * v[j];
     }
-    stf(out + t * C + c, acc);
+    stv<T, VEC>(out + t * C + c, acc);
 }
 
 // state <- the sequence's last K inputs after this chunk (thread per
@@ -256,12 +321,23 @@ extern "C" void launch_scalar_rmsnorm(const float* x, void* y, long T, int W,
                                       float gain, float eps, int out_f32,
                                       hipStream_t s) {
     if (T == 0) return;
-    const int th = row_threads(W);
     const size_t sh = (size_t)W * sizeof(float);
+    if (W % 4 == 0) {
+        const int th = row_threads(W / 4);
+        if (out_f32)
+            scalar_rmsnorm_kernel<float, 4><<<T, th, sh, s>>>(
+                x, (float*)y, W, gain, eps);
+        else
+            scalar_rmsnorm_kernel<unsigned short, 4><<<T, th, sh, s>>>(
+                x, (unsigned short*)y, W, gain, eps);
+        return;
+    }
+    const int th = row_threads(W);
     if (out_f32)
-        scalar_rmsnorm_kernel<float><<<T, th, sh, s>>>(x, (float*)y, W, gain, eps);
+        scalar_rmsnorm_kernel<float, 1><<<T, th, sh, s>>>(
+            x, (float*)y, W, gain, eps);
     else
-        scalar_rmsnorm_kernel<unsigned short><<<T, th, sh, s>>>(
+        scalar_rmsnorm_kernel<unsigned short, 1><<<T, th, sh, s>>>(
             x, (unsigned short*)y, W, gain, eps);
 }
 
@@ -269,13 +345,24 @@ template <typename YT, typename OT>
 static void add_norm_dispatch(float* resid, const void* y, const void* y2,
                               void* out, long T, int W, float post, float pre,
                               float eps, hipStream_t s) {
-    const int th = row_threads(W);
     const size_t sh = (size_t)W * sizeof(float);
+    if (W % 4 == 0) {
+        const int th = row_threads(W / 4);
+        if (out)
+            add_scalar_rmsnorm_kernel<YT, OT, true, 4><<<T, th, sh, s>>>(
+                resid, (const YT*)y, (const YT*)y2, (OT*)out, W, post, pre, eps);
+        else
+            add_scalar_rmsnorm_kernel<YT, OT, false, 4><<<T, th, sh, s>>>(
+                resid, (const YT*)y, (const YT*)y2, (OT*)nullptr, W, post, pre,
+                eps);
+        return;
+    }
+    const int th = row_threads(W);
     if (out)
-        add_scalar_rmsnorm_kernel<YT, OT, true><<<T, th, sh, s>>>(
+        add_scalar_rmsnorm_kernel<YT, OT, true, 1><<<T, th, sh, s>>>(
             resid, (const YT*)y, (const YT*)y2, (OT*)out, W, post, pre, eps);
     else
-        add_scalar_rmsnorm_kernel<YT, OT, false><<<T, th, sh, s>>>(
+        add_scalar_rmsnorm_kernel<YT, OT, false, 1><<<T, th, sh, s>>>(
             resid, (const YT*)y, (const YT*)y2, (OT*)nullptr, W, post, pre, eps);
 }
 
@@ -333,18 +420,32 @@ extern "C" void launch_canon_conv(const void* h, const float* w, void* state,
                                   int f32, hipStream_t s) {
     if (T == 0) return;
     const int th = C >= 256 ? 256 : 64;
-    const dim3 g1((unsigned)T, (C + th - 1) / th), g2(B, (C + th - 1) / th);
+    const int vec = C % 4 == 0 ? 4 : 1;
+    const int lanes = (C + vec - 1) / vec;
+    const dim3 g1((unsigned)T, (lanes + th - 1) / th), g2(B, (C + th - 1) / th);
     if (f32) {
-        canon_conv_kernel<float><<<g1, th, 0, s>>>(
-            (const float*)h, w, (const float*)state, state_slots, cu, seq_idx,
-            positions, (float*)out, C, K);
+        if (vec == 4)
+            canon_conv_kernel<float, 4><<<g1, th, 0, s>>>(
+                (const float*)h, w, (const float*)state, state_slots, cu,
+                seq_idx, positions, (float*)out, C, K);
+        else
+            canon_conv_kernel<float, 1><<<g1, th, 0, s>>>(
+                (const float*)h, w, (const float*)state, state_slots, cu, seq_idx,
+                positions, (float*)out, C, K);
         if (K > 0)
             canon_state_kernel<float><<<g2, th, 0, s>>>(
                 (const float*)h, (float*)state, state_slots, cu, C, K);
     } else {
-        canon_conv_kernel<unsigned short><<<g1, th, 0, s>>>(
-            (const unsigned short*)h, w, (const unsigned short*)state,
-            state_slots, cu, seq_idx, positions, (unsigned short*)out, C, K);
+        if (vec == 4)
+            canon_conv_kernel<unsigned short, 4><<<g1, th, 0, s>>>(
+                (const unsigned short*)h, w, (const unsigned short*)state,
+                state_slots, cu, seq_idx, positions, (unsigned short*)out, C,
+                K);
+        else
+            canon_conv_kernel<unsigned short, 1><<<g1, th, 0, s>>>(
+                (const unsigned short*)h, w, (const unsigned short*)state,
+                state_slots, cu, seq_idx, positions, (unsigned short*)out, C,
+                K);
         if (K > 0)
             canon_state_kernel<unsigned short><<<g2, th, 0, s>>>(
                 (const unsigned short*)h, (unsigned short*)state, state_slots,

@@ -48,7 +48,7 @@ def batch_meta(lens, starts, block_size, n_blocks, seed=0):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("W", [48, 200, 1024])
+@pytest.mark.parametrize("W", [37, 48, 200, 1024, 4096])
 def test_scalar_norms(dtype, W):
     torch.manual_seed(0)
     x = torch.randn(7, W, device=DEV) * 3
@@ -87,9 +87,9 @@ def test_gated_norm_and_glu(dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("taps", [1, 2, 4])
-def test_canon_conv_chunks_and_state(dtype, taps):
+@pytest.mark.parametrize("C", [72, 73, 1024])
+def test_canon_conv_chunks_and_state(dtype, taps, C):
     torch.manual_seed(2)
-    C = 72
     m = batch_meta([5, 1, 2, 9], [0, 7, 1, 30], 16, 16)
     h = torch.randn(m["T"], C, device=DEV).to(dtype)
     w = torch.randn(C, taps, device=DEV) * 0.3
