@@ -58,7 +58,7 @@ class LayerWeights:
         self.moe_w_gate_up = None
         self.moe_w_down = None
         self.gains = None      # (pre-mixer, post-mixer, pre-ffn, post-ffn)
-        self.canon = None      # [width, taps] fp32
+        self.canon = None      # [taps, width] fp32 (tap-major)
         self.kv_norm = None    # [kv_rank] fp32
         self.w_uk = None       # [heads, dim, kv_rank]
         self.w_uv = None       # [heads, kv_rank, vdim]
@@ -499,7 +499,8 @@ class ModelWeights:
                 if (f is not None or n in ("norm1", "norm1b")) else 1.0
                 for n in ("norm1", "norm1b", "norm2", "norm2b"))
             if s.canon_taps:
-                lw.canon = f32(get(p + "canon1"))
+                # checkpoint [width, taps] -> tap-major [taps, width]
+                lw.canon = f32(get(p + "canon1").t())
             if m.kind == "latent_attention":
                 # fused input projection rows: [q | latent+rot key | gate]
                 lw.wqkv = act(torch.cat([get(p + "mix.q"), get(p + "mix.dkv"),
@@ -631,7 +632,7 @@ def _save_nukopel(weights: "ModelWeights", out_dir: str, tensors, cpu) -> None:
         for n, g in zip(names, lw.gains):
             gain(p + n, g)
         if lw.canon is not None:
-            put(p + "canon1", lw.canon)
+            put(p + "canon1", lw.canon.t())
         H = m.heads
         if m.kind == "latent_attention":
             q, dkv, g = torch.split(

@@ -195,12 +195,12 @@ __global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ y,
 }
 
 // ------------------------------------------------------- input convolution
-// out[t] = h[t] + sum_d w[c][K-d] * h[t-d], d = 0..K (K = taps-1). Rows
+// out[t] = h[t] + sum_d w[K-d][c] * h[t-d], d = 0..K (K = taps-1). Rows
 // before the chunk come from the sequence's state (its last K inputs), rows
 // before position 0 are zero.
 template <typename T, int VEC>
 __global__ void canon_conv_kernel(const T* __restrict__ h,
-                                  const float* __restrict__ w,   // [C, K+1]
+                                  const float* __restrict__ w,   // [K+1, C]
                                   const T* __restrict__ state,   // [S, K, C]
                                   const int* __restrict__ state_slots,
                                   const int* __restrict__ cu,
@@ -214,11 +214,11 @@ __global__ void canon_conv_kernel(const T* __restrict__ h,
     const int local = (int)t - cu[b];
     const int pos = positions[t];
     const long slot = state_slots[b];
-    float acc[VEC], v[VEC];
+    float acc[VEC], v[VEC], wv[VEC];
     ldv<T, VEC>(h + t * C + c, v);
+    ldv<float, VEC>(w + (long)K * C + c, wv);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j)
-        acc[j] = v[j] * (1.f + w[(long)(c + j) * (K + 1) + K]);
+    for (int j = 0; j < VEC; ++j) acc[j] = v[j] * (1.f + wv[j]);
     for (int d = 1; d <= K; ++d) {
         if (pos - d < 0) break;
         const int src = local - d;
@@ -226,9 +226,9 @@ __global__ void canon_conv_kernel(const T* __restrict__ h,
             ldv<T, VEC>(h + (t - d) * C + c, v);
         else
             ldv<T, VEC>(state + (slot * K + (K + src)) * C + c, v);
+        ldv<float, VEC>(w + (long)(K - d) * C + c, wv);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j)
-            acc[j] += w[(long)(c + j) * (K + 1) + K - d] * v[j];
+        for (int j = 0; j < VEC; ++j) acc[j] += wv[j] * v[j];
     }
     stv<T, VEC>(out + t * C + c, acc);
 }

@@ -159,9 +159,9 @@ Tensor canon_conv(const Tensor& h, const Tensor& w, Tensor& state,
     check_i32(positions, "positions");
     TORCH_CHECK(h.dim() == 2 && h.is_contiguous());
     const long T = h.size(0);
-    const int C = (int)h.size(1), K = (int)w.size(1) - 1;
-    TORCH_CHECK(w.dim() == 2 && w.size(0) == C && K >= 0 && K <= 8,
-                "conv weight must be [channels, taps] with taps <= 9");
+    const int C = (int)h.size(1), K = (int)w.size(0) - 1;
+    TORCH_CHECK(w.dim() == 2 && w.size(1) == C && K >= 0 && K <= 8,
+                "conv weight must be [taps, channels] with taps <= 9");
     const int B = (int)cu.numel() - 1;
     TORCH_CHECK(state_slots.numel() == B && seq_idx.numel() == T &&
                 positions.numel() == T);

@@ -347,14 +347,15 @@ def add_scalar_rmsnorm(resid: torch.Tensor, y: torch.Tensor, post_gain: float,
 def canon_conv(h: torch.Tensor, w: torch.Tensor, state: torch.Tensor,
                state_slots: torch.Tensor, cu_seqlens: torch.Tensor,
                seq_idx: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
-    """h + causal per-channel conv over time. h [T, C]; w [C, taps] (tap
-    taps-1 multiplies the current row); state [n_slots, taps-1, C] holds each
-    sequence's last taps-1 inputs and is advanced in place."""
+    """h + causal per-channel conv over time. h [T, C]; w [taps, C],
+    tap-major (row taps-1 multiplies the current input, row 0 the oldest);
+    state [n_slots, taps-1, C] holds each sequence's last taps-1 inputs and
+    is advanced in place."""
     T, C = h.shape
-    K = w.shape[1] - 1
+    K = w.shape[0] - 1
     wf = w.float()
     hf = h.float()
-    out = hf * (1.0 + wf[:, K])
+    out = hf * (1.0 + wf[K])
     if K == 0:
         return out.to(h.dtype)
     sidx = seq_idx.long()
@@ -370,7 +371,7 @@ def canon_conv(h: torch.Tensor, w: torch.Tensor, state: torch.Tensor,
         val = torch.where(in_chunk[:, None], from_chunk, from_state)
         # select, never multiply: a reused slot may hold anything
         val = torch.where((pos - d >= 0)[:, None], val, torch.zeros_like(val))
-        out += wf[:, K - d] * val
+        out += wf[K - d] * val
     # advance the state: the last K inputs of each sequence after this chunk
     cu = cu_seqlens.long()
     B = cu.numel() - 1

@@ -92,7 +92,7 @@ def test_canon_conv_chunks_and_state(dtype, taps, C):
     torch.manual_seed(2)
     m = batch_meta([5, 1, 2, 9], [0, 7, 1, 30], 16, 16)
     h = torch.randn(m["T"], C, device=DEV).to(dtype)
-    w = torch.randn(C, taps, device=DEV) * 0.3
+    w = torch.randn(taps, C, device=DEV) * 0.3
     st = torch.randn(6, max(taps - 1, 0), C, device=DEV).to(dtype)
     st1, st2 = st.clone(), st.clone()
     o1 = ops.canon_conv(h, w, st1, m["state_slots"], m["cu"], m["seq"], m["pos"])

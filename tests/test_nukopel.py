@@ -55,7 +55,8 @@ def test_conv_portions_carry_state(taps, cuts):
     state = torch.full((3, taps - 1, C), float("nan"))
     got, at = [], 0
     for n in cuts:
-        got.append(ref.canon_conv(h[at:at + n], w, state, i32([2]),
+        got.append(ref.canon_conv(h[at:at + n], w.t().contiguous(), state,
+                                  i32([2]),
                                   i32([0, n]), i32([0] * n),
                                   i32(list(range(at, at + n)))))
         at += n
@@ -80,8 +81,8 @@ def test_conv_batch_of_unequal_chunks():
             cu.append(cu[-1] + n)
             sidx += [b] * n
             pos += list(range(at[b], at[b] + n))
-        o = ref.canon_conv(torch.cat(hs), w, state, slots, i32(cu), i32(sidx),
-                           i32(pos))
+        o = ref.canon_conv(torch.cat(hs), w.t().contiguous(), state, slots,
+                           i32(cu), i32(sidx), i32(pos))
         for b, n in enumerate(takes):
             outs[b].append(o[cu[b]:cu[b + 1]])
             at[b] += n
