@@ -394,18 +394,21 @@ latent_attn_mfma_kernel(const unsigned short* __restrict__ q_abs,
     }
 }
 
-// merge the key-split partials of one (token, head): one wave per row.
-// Lane z < splits holds share z's (max, sum); the merge weights
-// exp(m_z - M) are computed once and broadcast by shuffle.
+// merge the key-split partials of one (token, head): one workgroup per row.
+// In every wave, lane z < splits holds share z's (max, sum); the merge
+// weights exp(m_z - M) are computed once per wave and broadcast by shuffle,
+// and each thread merges its columns with `splits` independent loads.
+constexpr int LC_THREADS = 256;
+
 template <typename T>
-__global__ void __launch_bounds__(WAVE)
+__global__ void __launch_bounds__(LC_THREADS)
 latent_attn_combine_kernel(const float* __restrict__ part_acc,
                            const float* __restrict__ part_ml,
                            const T* __restrict__ gate, long gate_tok,
                            T* __restrict__ out, int splits, int Tn, int H,
                            int C) {
     const int t = blockIdx.x, h = blockIdx.y;
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x % WAVE;
     float m = -INFINITY, l = 0.f;
     if (lane < splits) {
         const long row = ((long)lane * H + h) * Tn + t;
@@ -419,8 +422,8 @@ latent_attn_combine_kernel(const float* __restrict__ part_acc,
     const float r = g / L;
     T* o = out + ((long)h * Tn + t) * C;
     // uniform trip count: every lane takes part in every shuffle
-    for (int c0 = 0; c0 < C; c0 += WAVE) {
-        const int c = c0 + lane;
+    for (int c0 = 0; c0 < C; c0 += LC_THREADS) {
+        const int c = c0 + threadIdx.x;
         float a = 0.f;
         for (int z = 0; z < splits; ++z) {
             const float wz = __shfl(w, z);
@@ -644,7 +647,7 @@ static int latent_attn_dispatch(const void* q_abs, const void* q_rot,
     }
     if (splits > 1) {
         const dim3 g2(Tn, H);
-        latent_attn_combine_kernel<TT><<<g2, WAVE, 0, s>>>(
+        latent_attn_combine_kernel<TT><<<g2, LC_THREADS, 0, s>>>(
             part_acc, part_ml, (const TT*)gate, gate_tok, (TT*)out, splits,
             Tn, H, C);
     }
@@ -707,7 +710,7 @@ extern "C" int launch_latent_attn_mfma(
         if (splits > 1) {
             const dim3 g2(Tn, H);
             latent_attn_combine_kernel<unsigned short>
-                <<<g2, WAVE, 0, s>>>(
+                <<<g2, LC_THREADS, 0, s>>>(
                     part_acc, part_ml, (const unsigned short*)gate, gate_tok,
                     (unsigned short*)out, splits, Tn, H, C);
         }
