@@ -5,15 +5,18 @@ and write the logits at chosen places. Nothing is sampled.
 
 Steps arrive on standard input, one JSON object a line:
 
-    {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}],
-     "end": []}
+    {"step": 7, "entries": [{"id": "req-1", "tokens": [41, 8], "want": [1]},
+                            {"id": "req-2", "tokens": [300], "want": []}],
+     "end": ["req-2"]}
 
-All entries of a step run as one packed batch through the engine's chunk
-forward (InferenceEngine.feed): portions of prompts beside single decoded
-tokens, against the pages and state slots that earlier steps left. For a
-step in which something is wanted, OUT/<step>.f32 receives the logits at
-the wanted places (entry order, then `want` order) as little-endian fp32
-[wanted, vocab]; after every step the line `done <step>` is printed.
+`entries` bring each request's next tokens and the indices (`want`) among
+them whose logits to report; `end` names requests that release their pages
+and state slot after the step. The entries of a step form one packed batch
+through the engine's chunk forward (InferenceEngine.feed) — prompt portions
+next to single decode tokens — continuing from whatever earlier steps left
+in the cache. Logits go to OUT/<step>.f32 (rows in entry order, then `want`
+order; little-endian fp32, [rows, vocab]) when a step wants any, and every
+step is acknowledged with a flushed `done <step>` line on standard output.
 
 The engine is built with a page pool for --max-tokens tokens (each live
 request rounded up to whole pages) and state slots for four requests, so
