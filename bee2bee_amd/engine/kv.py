@@ -12,10 +12,16 @@ the SAME page and slot bookkeeping:
   * latent-attention layers: one page pool [n_blocks, block_size,
     kv_rank + rot_dim] — the normed latent and the shared rotated key part
     of each token (k_cache[i]; there is no separate value pool);
-  * linear-attention layers: no pages, a recurrent state
-    [n_slots, heads, dim, vdim] fp32 per sequence slot;
-  * every layer with an input convolution: the last taps-1 mixer inputs
-    [n_slots, taps-1, width] per sequence slot.
+  * sink-attention layers (grouped-query softmax attention whose values
+    are the raw key projection): the dense page layout, k_cache[i] holding
+    normed+rotated keys and v_cache[i] the keys as projected;
+  * linear-attention / retention / delta-rule layers: no pages, a recurrent
+    state [n_slots, heads, dim, vdim] fp32 per sequence slot;
+  * every layer with a convolution: the last taps-1 conv inputs
+    [n_slots, taps-1, channels] per sequence slot (the mixer input for the
+    whole-width conv, the q|k|v projection for a delta mixer's short conv);
+  * a parallel mixer (attention + delta rule side by side) has pages AND
+    state in the same layer.
 A sequence owns one state slot from new_seq to free_seq. Slots and pages
 are handed out again without clearing: the kernels never read state or
 cache rows that precede a sequence's position 0.
@@ -91,20 +97,39 @@ class PagedKV:
         self.k_cache, self.v_cache = [], []
         self.conv_state: List[Optional[torch.Tensor]] = []
         self.rec_state: List[Optional[torch.Tensor]] = []
+        from ..models.hybrid import mixer_parts
+
         taps = spec.canon_taps
+        f32 = torch.float32
         for l in spec.layer_specs:
-            m = l.mixer
-            latent = m.kind == "latent_attention"
-            self.k_cache.append(torch.zeros(
-                self.n_blocks, self.block_size, m.cache_dim, device=dev,
-                dtype=self.dtype) if latent else None)
-            self.v_cache.append(None)
-            self.rec_state.append(None if latent else torch.zeros(
-                n_slots, m.heads, m.dim, m.vdim, device=dev,
-                dtype=torch.float32))
-            self.conv_state.append(torch.zeros(
-                n_slots, taps - 1, spec.hidden_size, device=dev,
-                dtype=self.dtype) if taps >= 1 else None)
+            k = v = rec = conv = None
+            for _, m in mixer_parts(l.mixer):
+                if m.kind == "latent_attention":
+                    k = torch.zeros(self.n_blocks, self.block_size,
+                                    m.cache_dim, device=dev, dtype=self.dtype)
+                elif m.kind == "sink_attention":
+                    # the dense models' page layout: one (key, head) row
+                    # contiguous; values here are the raw key projection
+                    k = torch.zeros(self.n_blocks, m.kv_heads,
+                                    self.block_size, m.dim, device=dev,
+                                    dtype=self.dtype)
+                    v = torch.zeros(self.n_blocks, m.kv_heads,
+                                    self.block_size, m.vdim, device=dev,
+                                    dtype=self.dtype)
+                else:   # lightning / retention / delta: recurrent state
+                    rec = torch.zeros(n_slots, m.heads, m.dim, m.vdim,
+                                      device=dev, dtype=f32)
+                    if m.kind == "delta" and m.taps > 1:
+                        conv = torch.zeros(n_slots, m.taps - 1,
+                                           m.conv_channels, device=dev,
+                                           dtype=self.dtype)
+            if l.form == "sandwich" and taps >= 1:
+                conv = torch.zeros(n_slots, taps - 1, spec.hidden_size,
+                                   device=dev, dtype=self.dtype)
+            self.k_cache.append(k)
+            self.v_cache.append(v)
+            self.rec_state.append(rec)
+            self.conv_state.append(conv)
 
     # ------------------------------------------------------- state slots
 

@@ -89,6 +89,12 @@ class Runner:
         return ops.fused_add_rmsnorm(x, resid, w, self.spec.rms_eps)
 
     def lm_head(self, hidden: torch.Tensor) -> torch.Tensor:
+        if self.spec.is_hybrid and self.weights.final_gain is None:
+            # fp32 residual stream, weighted final norm
+            normed = ops.rmsnorm_f32(
+                hidden.contiguous(), self.weights.final_norm,
+                self.spec.rms_eps, self.dtype)
+            return F.linear(normed, self.weights.lm_head)
         if self.spec.is_hybrid:
             # hidden is the fp32 residual stream; scalar-gain final norm
             normed = ops.scalar_rmsnorm(
@@ -402,11 +408,14 @@ class Runner:
 
     # --------------------------------------------------------- hybrid stacks
 
-    def _rope_tables(self, dims: int, base: float):
-        key = (dims, base)
+    def _rope_tables(self, dims: int, base: float, f64: bool = False):
+        """cos/sin tables per (dims, base); f64: angles evaluated in float64
+        before the single rounding to fp32."""
+        key = (dims, base, f64)
         t = self._rope_by_cfg.get(key)
         if t is None:
-            t = ops.rope_tables(self.spec.max_seq_len, dims, base, self.device)
+            make = ops.rope_tables_f64 if f64 else ops.rope_tables
+            t = make(self.spec.max_seq_len, dims, base, self.device)
             self._rope_by_cfg[key] = t
         return t
 
@@ -443,9 +452,21 @@ class Runner:
         x = F.embedding(input_ids, W.embed).float()
         if s.embed_scale != 1.0:
             x = x * s.embed_scale
+        n = s.n_layers
+        if s.layer_specs[0].form == "parallel":
+            # x += mixer(h) + ffn(h), h = unit(x) * w: the residual add and
+            # the next layer's norm run as one kernel
+            eps, dt = s.rms_eps, self.dtype
+            normed = ops.rmsnorm_f32(x, W.layers[0].norm_w, eps, dt)
+            for i in range(n):
+                y = self._parallel_layer(i, normed, meta)
+                nxt = W.layers[i + 1].norm_w if i + 1 < n else None
+                normed = ops.add_rmsnorm_f32(x, y, nxt, eps, dt)
+                if self.layer_tap is not None:
+                    self.layer_tap(i, x)
+            return x
         normed = ops.scalar_rmsnorm(x, W.layers[0].gains[0], s.rms_eps,
                                     self.dtype)
-        n = s.n_layers
         for i in range(n):
             nxt = W.layers[i + 1].gains[0] if i + 1 < n else None
             normed = self._hybrid_layer(i, x, normed, meta, nxt)
@@ -511,3 +532,100 @@ class Runner:
                           lw.w_down)
         return ops.add_scalar_rmsnorm(x, y, lw.gains[3], next_gain, eps, dt,
                                       y2=y2)
+
+    # ------------------------------------------------- parallel-form layers
+
+    def _parallel_layer(self, i: int, h: torch.Tensor, meta) -> torch.Tensor:
+        """mixer(h) + ffn(h) of layer i as two GEMMs: one input projection
+        for everything that reads h (the feed-forward's up included), the
+        mixer kernels and the activation writing column slices of ONE
+        buffer, and one output projection over that buffer, which sums the
+        mixer parts and the feed-forward in its fp32 accumulator."""
+        from ..models.hybrid import mixer_parts
+
+        s = self.spec
+        lw, l = self.weights.layers[i], s.layer_specs[i]
+        ins, n_in, outs, n_out = lw.layout
+        T = h.shape[0]
+        proj = F.linear(h, lw.w_in)                         # [T, n_in]
+        exact = n_out == sum(n for _, n in outs.values())
+        buf = (torch.empty if exact else torch.zeros)(
+            T, n_out, dtype=self.dtype, device=h.device)
+
+        def cols(key):
+            off, n = ins[key]
+            return proj[:, off : off + n]
+
+        m = l.mixer
+        for pre, part in mixer_parts(m):
+            scale = 1.0
+            if m.kind == "parallel":
+                scale = m.left_scale if pre == "left." else m.right_scale
+            off, n = outs[pre + "o"]
+            out = buf[:, off : off + n]
+            ns = lw.mix[pre]
+            if part.kind == "retention":
+                self._retention_part(i, part, ns, cols, pre, meta, out, scale)
+            elif part.kind == "delta":
+                self._delta_part(i, part, ns, cols, pre, meta, out, scale)
+            else:
+                self._sink_attn_part(i, part, ns, cols, pre, meta, out, scale)
+        if l.ffn is not None:
+            off, n = outs["down"]
+            ops.relu2(cols("up"), buf[:, off : off + n])
+        return F.linear(buf, lw.w_out)
+
+    def _retention_part(self, i, m, ns, cols, pre, meta, out, scale) -> None:
+        positions, _, cu, _, _, state_slots, max_qlen = meta
+        T, H = positions.shape[0], m.heads
+        cos = sin = None
+        if m.rope_dims:
+            cos, sin = self._rope_tables(m.rope_dims, m.rope_base, f64=True)
+        o = ops.retention_attn(
+            cols(pre + "q").view(T, H, m.dim), cols(pre + "k").view(T, H, m.dim),
+            cols(pre + "v").view(T, H, m.vdim), ns.decay, m.rope_dims, cos,
+            sin, m.dim ** -0.5, self.kv.rec_state[i], state_slots, cu,
+            positions, max_qlen)
+        ops.head_gated_norm(o.view(T, H, m.vdim), None, cols(pre + "g"),
+                            "silu", self.spec.rms_eps, out, scale)
+
+    def _delta_part(self, i, m, ns, cols, pre, meta, out, scale) -> None:
+        positions, _, cu, seq_idx, _, state_slots, _ = meta
+        T, H, G, D = positions.shape[0], m.heads, m.kv_heads, m.dim
+        conv_state = self.kv.conv_state[i]
+        if conv_state is None:       # a single tap carries nothing
+            conv_state = out.new_empty(0)
+        qkv = ops.short_conv(cols(pre + "qkv"), ns.conv_w, conv_state,
+                             state_slots, cu, seq_idx, positions, True)
+        a = cols(pre + "a")
+        if ns.a2 is not None:
+            a = F.linear(a, ns.a2)
+        beta, g = ops.delta_gates(qkv, G, D, cols(pre + "b"), a, ns.dt_bias,
+                                  ns.rate, m.channel_decay)
+        nq = G * D
+        o = ops.delta_rule(
+            qkv[:, :nq].view(T, G, D), qkv[:, nq : 2 * nq].view(T, G, D),
+            qkv[:, 2 * nq :].view(T, H, m.vdim), beta, g,
+            self.kv.rec_state[i], state_slots, cu, positions)
+        gate = cols(pre + "g")
+        if ns.g2 is not None:
+            gate = F.linear(gate, ns.g2)
+        ops.head_gated_norm(o, ns.norm, gate, m.gate, self.spec.rms_eps, out,
+                            scale)
+
+    def _sink_attn_part(self, i, m, ns, cols, pre, meta, out, scale) -> None:
+        (positions, slot_mapping, cu, seq_idx, block_table, _,
+         max_qlen) = meta
+        T = positions.shape[0]
+        q = cols(pre + "q").view(T, m.heads, m.dim)
+        k = cols(pre + "k").view(T, m.kv_heads, m.dim)
+        cos = sin = None
+        if m.rope_dims:
+            cos, sin = self._rope_tables(m.rope_dims, m.rope_base, f64=True)
+        k_cache, v_cache = self.kv.k_cache[i], self.kv.v_cache[i]
+        # q leaves this with every score multiplier folded in
+        ops.qk_norm_rope_store(q, k, ns.q_norm, ns.k_norm, self.spec.rms_eps,
+                               m.rope_dims, positions, cos, sin, ns.q_mult,
+                               k_cache, v_cache, slot_mapping)
+        ops.sink_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
+                      cu, ns.sink, m.window, out, scale, max_qlen)

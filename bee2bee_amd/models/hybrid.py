@@ -14,6 +14,14 @@ Nukopel config.json keys (the family served through this path):
   architecture, vocab, width, canon.taps, embedding.scale, norm.eps,
   layers[i].type in {latent_attention, lightning},
   layers[i].mixer.{heads, dim, vdim, ...}, layers[i].mlp (or null).
+
+Pugozen config.json keys (parallel-form layers: one weighted RMS norm whose
+output feeds the mixer AND the feed-forward, both added to the residual):
+  architecture, vocab, width, embedding.scale, norm.eps,
+  layers[i].type in {retention, delta, parallel}, layers[i].weights_of,
+  layers[i].mixer.{heads, kv_heads, dim, vdim, decay, conv, rot.{base,dims},
+  scale, left, right, left_scale, right_scale},
+  layers[i].mlp.{kind: dense, ff} (or null).
 """
 from __future__ import annotations
 
@@ -60,6 +68,128 @@ class LightningSpec:
 
 
 @dataclass
+class RetentionSpec:
+    """Linear attention with a fixed per-head decay, no softmax and no
+    denominator, on rotated queries/keys:
+    memory M (dim x vdim per head), M <- lam_h M + (k / sqrt(dim)) v^T per
+    token, read-out y = M^T q, then per-head unit norm (no weight) and a
+    silu output gate."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: Tuple[float, ...]
+    rope_base: float = 10000.0
+    rope_dims: int = 0      # leading dims of each head that rotate (0: none)
+
+    kind = "retention"
+
+    @property
+    def in_sizes(self) -> Tuple[Tuple[str, int], ...]:
+        """Rows of the fused input projection, in order."""
+        return (("q", self.heads * self.dim), ("k", self.heads * self.dim),
+                ("v", self.heads * self.vdim), ("g", self.heads * self.vdim))
+
+    @property
+    def out_size(self) -> int:
+        return self.heads * self.vdim
+
+
+@dataclass
+class DeltaSpec:
+    """Gated delta rule with a carried fp32 memory M (dim x vdim) per
+    head. Per token: fade M <- gamma * M; what the key already recalls is
+    taken out of the write, delta = beta (v - M^T k); M <- M + k delta^T;
+    read-out y = M^T q (it sees the token's own write).
+    q/k (kv_heads x dim, shared by groups of value heads) and v pass a short
+    causal per-channel convolution + silu; q, k are unit vectors.
+    channel_decay: gamma is one number per head (False: projection 'a') or one
+    per head and key channel (True: low-rank projection 'a2 a1').
+    gate: "silu" with a full projection 'g', or "sigmoid" with the low-rank
+    pair 'g2 g1'."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    taps: int
+    channel_decay: bool = False
+    decay_rank: int = 0
+    gate: str = "silu"
+    gate_rank: int = 0
+
+    kind = "delta"
+
+    @property
+    def conv_channels(self) -> int:
+        return 2 * self.kv_heads * self.dim + self.heads * self.vdim
+
+    @property
+    def in_sizes(self) -> Tuple[Tuple[str, int], ...]:
+        n_a = self.decay_rank if self.channel_decay else self.heads
+        n_g = self.gate_rank if self.gate_rank else self.heads * self.vdim
+        return (("qkv", self.conv_channels), ("b", self.heads), ("a", n_a),
+                ("g", n_g))
+
+    @property
+    def out_size(self) -> int:
+        return self.heads * self.vdim
+
+
+@dataclass
+class SinkAttnSpec:
+    """Causal grouped-query softmax attention over paged keys with
+    per-head RMS-normed, partly rotated queries/keys, a per-head score
+    multiplier and a per-head sink logit in the softmax denominator (no key,
+    no value). value_from_key: the values ARE the key projection as
+    projected (before norm and rotation); there is no value projection.
+    window: 0 = every earlier position, else 0 <= i - j < window."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    rope_base: float = 10000.0
+    rope_dims: int = 0
+    window: int = 0
+    value_from_key: bool = True
+
+    kind = "sink_attention"
+
+    @property
+    def in_sizes(self) -> Tuple[Tuple[str, int], ...]:
+        return (("q", self.heads * self.dim), ("k", self.kv_heads * self.dim))
+
+    @property
+    def out_size(self) -> int:
+        return self.heads * self.vdim
+
+
+@dataclass
+class ParallelMixerSpec:
+    """Two mixers on the same input, summed with fixed scales."""
+    left: Any               # SinkAttnSpec
+    right: Any              # DeltaSpec
+    left_scale: float
+    right_scale: float
+
+    kind = "parallel"
+
+    @property
+    def heads(self) -> int:
+        return max(self.left.heads, self.right.heads)
+
+    @property
+    def dim(self) -> int:
+        return max(self.left.dim, self.right.dim)
+
+
+@dataclass
+class DenseFFNSpec:
+    """down(act(up h)); act "relu2" is the square of relu."""
+    ff: int
+    act: str = "relu2"
+
+
+@dataclass
 class MoEFFNSpec:
     """Routed experts (+ optional always-on shared expert) with the clamped
     GLU activation: g = min(gate, limit), u = clamp(up, +-limit),
@@ -75,8 +205,13 @@ class MoEFFNSpec:
 
 @dataclass
 class LayerSpec:
-    mixer: Any                      # LatentAttnSpec | LightningSpec
-    ffn: Optional[MoEFFNSpec] = None
+    mixer: Any                      # one of the mixer specs above
+    ffn: Any = None                 # MoEFFNSpec | DenseFFNSpec | None
+    # "sandwich": scalar-gain norms before and after each sublayer, mixer
+    # then feed-forward. "parallel": x += mixer(h) + ffn(h), h = norm(x) * w.
+    form: str = "sandwich"
+    # layer whose tensors this layer uses (its own cache and state)
+    weights_of: Optional[int] = None
 
     @property
     def kind(self) -> str:
@@ -101,7 +236,47 @@ def _mixer_from_cfg(kind: str, m: Dict[str, Any]):
             raise ValueError("lightning mixer needs one decay per head")
         return LightningSpec(heads=int(m["heads"]), dim=int(m["dim"]),
                              vdim=int(m["vdim"]), decay=decay)
+    rot = m.get("rot") or {}
+    if kind == "retention":
+        decay = tuple(float(d) for d in m["decay"])
+        if len(decay) != int(m["heads"]):
+            raise ValueError("retention mixer needs one decay per head")
+        return RetentionSpec(
+            heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+            decay=decay, rope_base=float(rot.get("base", 10000.0)),
+            rope_dims=int(rot.get("dims", 0)))
+    if kind == "delta":
+        return _delta_from_cfg(m, channel_decay=False, gate="silu")
+    if kind == "sink_attention":
+        return SinkAttnSpec(
+            heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
+            dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
+            scale=float(m["scale"]),
+            rope_base=float(rot.get("base", 10000.0)),
+            rope_dims=int(rot.get("dims", 0)))
+    if kind == "parallel":
+        return ParallelMixerSpec(
+            left=_mixer_from_cfg("sink_attention", m["left"]),
+            right=_delta_from_cfg(m["right"], channel_decay=True,
+                                  gate="sigmoid"),
+            left_scale=float(m["left_scale"]),
+            right_scale=float(m["right_scale"]))
     raise ValueError(f"unknown mixer type {kind!r}")
+
+
+def _delta_from_cfg(m: Dict[str, Any], channel_decay: bool,
+                    gate: str) -> DeltaSpec:
+    heads = int(m["heads"])
+    kv_heads = int(m.get("kv_heads", heads))
+    if heads % kv_heads:
+        raise ValueError("delta mixer: heads must be a multiple of kv_heads")
+    # low-rank widths are tensor shapes, not config keys: filled in by
+    # complete_from_shapes() (checkpoints) or given directly (synthetic)
+    return DeltaSpec(heads=heads, kv_heads=kv_heads, dim=int(m["dim"]),
+                     vdim=int(m["vdim"]), taps=int(m["conv"]),
+                     channel_decay=channel_decay, gate=gate,
+                     decay_rank=int(m.get("decay_rank", 0)),
+                     gate_rank=int(m.get("gate_rank", 0)))
 
 
 def _ffn_from_cfg(f: Optional[Dict[str, Any]]) -> Optional[MoEFFNSpec]:
@@ -123,11 +298,101 @@ def layer_specs_from_cfg(layers: List[Dict[str, Any]]) -> List[LayerSpec]:
                       ffn=_ffn_from_cfg(l.get("mlp"))) for l in layers]
 
 
+def parallel_layer_specs_from_cfg(layers: List[Dict[str, Any]]
+                                  ) -> List[LayerSpec]:
+    """Parallel-form layers (Pugozen): dense feed-forward, optional
+    'weights_of' (a layer that runs another layer's tensors)."""
+    out = []
+    for i, l in enumerate(layers):
+        f = l.get("mlp")
+        if f and f.get("kind", "dense") != "dense":
+            raise ValueError(f"unknown feed-forward kind {f.get('kind')!r}")
+        src = l.get("weights_of")
+        if src is not None:
+            # follow a chain to the layer that owns the tensors
+            src, hops = int(src), 0
+            while 0 <= src < len(layers) and \
+                    layers[src].get("weights_of") is not None:
+                src, hops = int(layers[src]["weights_of"]), hops + 1
+                if hops > len(layers):
+                    raise ValueError(f"layer {i}: weights_of forms a cycle")
+            if not 0 <= src < len(layers) or src == i:
+                raise ValueError(f"layer {i}: bad weights_of {src}")
+            if layers[src]["type"] != l["type"]:
+                raise ValueError(f"layer {i}: weights_of a layer of another type")
+        out.append(LayerSpec(
+            mixer=_mixer_from_cfg(l["type"], l["mixer"]),
+            ffn=DenseFFNSpec(ff=int(f["ff"])) if f else None,
+            form="parallel", weights_of=src))
+    return out
+
+
+def complete_from_shapes(layers: List[LayerSpec],
+                         shapes: Dict[str, Tuple[int, ...]]) -> None:
+    """Sizes that only tensor shapes give: the low-rank widths of a delta
+    mixer's decay and gate projections ('a1' / 'g1' rows)."""
+    for i, l in enumerate(layers):
+        src = i if l.weights_of is None else l.weights_of
+        m, p = l.mixer, f"l{src}.mix."
+        if m.kind == "parallel":
+            m, p = m.right, p + "right."
+        if m.kind != "delta":
+            continue
+        if m.channel_decay and p + "a1" in shapes:
+            m.decay_rank = int(shapes[p + "a1"][0])
+        if m.gate == "sigmoid" and p + "g1" in shapes:
+            m.gate_rank = int(shapes[p + "g1"][0])
+
+
+def _pad8(n: int) -> int:
+    return (n + 7) // 8 * 8
+
+
+def mixer_parts(m) -> List[Tuple[str, Any]]:
+    """(tensor-name prefix, sub-mixer) of a mixer: itself, or the two sides
+    of a parallel mixer."""
+    if m.kind == "parallel":
+        return [("left.", m.left), ("right.", m.right)]
+    return [("", m)]
+
+
+def fused_layout(l: LayerSpec) -> Tuple[Dict[str, Tuple[int, int]], int,
+                                        Dict[str, Tuple[int, int]], int]:
+    """Column layout of a parallel-form layer's two fused GEMMs.
+    Input side: every projection that reads the normed h — the mixer's
+    (per part, in in_sizes order) and the feed-forward's 'up' — stacked into
+    one [rows, width] matrix. Output side: the mixer parts' outputs and the
+    feed-forward activation laid side by side as the K axis of one
+    [width, K] matrix, so mixer + feed-forward are summed inside the GEMM's
+    fp32 accumulator. Every segment starts on a multiple of 8 elements
+    (16-byte aligned rows for bf16). Returns (in {name: (offset, size)},
+    in_total, out {name: (offset, size)}, out_total)."""
+    ins: Dict[str, Tuple[int, int]] = {}
+    outs: Dict[str, Tuple[int, int]] = {}
+    a = b = 0
+    for pre, m in mixer_parts(l.mixer):
+        for name, n in m.in_sizes:
+            ins[pre + name] = (a, n)
+            a += _pad8(n)
+        outs[pre + "o"] = (b, m.out_size)
+        b += _pad8(m.out_size)
+    if l.ffn is not None:
+        ins["up"] = (a, l.ffn.ff)
+        a += _pad8(l.ffn.ff)
+        outs["down"] = (b, l.ffn.ff)
+        b += _pad8(l.ffn.ff)
+    return ins, a, outs, b
+
+
 def hybrid_n_params(width: int, vocab: int, taps: int,
                     layers: List[LayerSpec], active_only: bool = False) -> int:
     n = 2 * vocab * width + 1
     for l in layers:
         m = l.mixer
+        if l.form == "parallel":
+            if l.weights_of is None or active_only:
+                n += width + _parallel_layer_params(width, l)
+            continue
         n += 4 + width * taps
         if m.kind == "latent_attention":
             n += width * (m.q_size + m.cache_dim + m.heads) + m.kv_rank
@@ -140,6 +405,61 @@ def hybrid_n_params(width: int, vocab: int, taps: int,
             e = f.top_k if active_only else f.n_experts
             n += width * f.n_experts + 3 * width * (e * f.ff + f.shared_ff)
     return n
+
+
+def _parallel_layer_params(width: int, l: LayerSpec) -> int:
+    n = 0
+    for _, m in mixer_parts(l.mixer):
+        n += width * m.out_size
+        if m.kind == "retention":
+            n += width * sum(sz for _, sz in m.in_sizes)
+        elif m.kind == "sink_attention":
+            n += width * sum(sz for _, sz in m.in_sizes) + 2 * m.dim + 2 * m.heads
+        else:
+            n += (width + m.taps) * m.conv_channels + width * m.heads
+            n += m.heads + m.vdim
+            hd = m.heads * m.dim
+            n += (m.decay_rank * (width + hd) + hd if m.channel_decay
+                  else (width + 1) * m.heads)
+            hv = m.heads * m.vdim
+            n += m.gate_rank * (width + hv) if m.gate_rank else width * hv
+    if l.ffn is not None:
+        n += 2 * width * l.ffn.ff
+    return n
+
+
+def pugozen_layers(n_layers: int, width: int, *, heads: int = 16,
+                   kv_heads: int = 4, dim: int = 128, ff: int = 8192,
+                   delta_heads: int = 16, delta_kv_heads: int = 8,
+                   delta_dim: int = 128, rank: int = 64, taps: int = 4,
+                   side_heads: int = 4, side_dim: int = 64
+                   ) -> List[LayerSpec]:
+    """A synthetic Pugozen stack for benchmarks: the cycle
+    parallel / retention / delta, all with a dense relu^2 feed-forward."""
+    out = []
+    for i in range(n_layers):
+        k = i % 3
+        if k == 0:
+            mixer: Any = ParallelMixerSpec(
+                left=SinkAttnSpec(heads=heads, kv_heads=kv_heads, dim=dim,
+                                  vdim=dim, scale=dim ** -0.5, rope_base=1e6,
+                                  rope_dims=dim // 2),
+                right=DeltaSpec(heads=side_heads, kv_heads=side_heads,
+                                dim=side_dim, vdim=side_dim, taps=taps,
+                                channel_decay=True, decay_rank=rank,
+                                gate="sigmoid", gate_rank=rank),
+                left_scale=0.75, right_scale=0.5)
+        elif k == 1:
+            decay = tuple(1.0 - 2.0 ** (-5.0 - 3.0 * h / max(1, heads - 1))
+                          for h in range(heads))
+            mixer = RetentionSpec(heads=heads, dim=dim, vdim=dim, decay=decay,
+                                  rope_base=1e6, rope_dims=dim)
+        else:
+            mixer = DeltaSpec(heads=delta_heads, kv_heads=delta_kv_heads,
+                              dim=delta_dim, vdim=delta_dim, taps=taps)
+        out.append(LayerSpec(mixer=mixer, ffn=DenseFFNSpec(ff=ff),
+                             form="parallel"))
+    return out
 
 
 def nukopel_layers(n_layers: int, width: int, *, attn_every: int = 4,

@@ -48,7 +48,7 @@ class ModelSpec:
     # vocab specials (byte-tokenizer defaults; overridden by a real tokenizer)
     bos_token_id: int = 1
     eos_token_id: int = 2
-    # hybrid stacks (arch "nukopel"): per-layer mixer/feed-forward specs
+    # hybrid stacks (arch "nukopel", "pugozen"): per-layer mixer/feed-forward specs
     # (models/hybrid.py). When set, the uniform-layer fields above hold
     # representative maxima only; the Runner's hybrid path reads these.
     layer_specs: Optional[List[Any]] = None
@@ -415,7 +415,9 @@ _ALIASES = {
 
 def hybrid_spec(name: str, vocab: int, width: int, layer_specs: List[Any],
                 *, eps: float, embed_scale: float, canon_taps: int,
-                max_seq_len: int = 32768) -> ModelSpec:
+                max_seq_len: int = 32768, arch: str = "nukopel",
+                norm_type: str = "scalar_rmsnorm",
+                act_type: str = "clamped_glu") -> ModelSpec:
     """ModelSpec for a hybrid stack (models/hybrid.py layer specs)."""
     ffns = [l.ffn for l in layer_specs if l.ffn is not None]
     return ModelSpec(
@@ -426,9 +428,9 @@ def hybrid_spec(name: str, vocab: int, width: int, layer_specs: List[Any],
         n_kv_heads=1,
         head_dim=max(l.mixer.dim for l in layer_specs),
         rms_eps=eps, max_seq_len=max_seq_len, tie_embeddings=False,
-        n_experts=max([f.n_experts for f in ffns] or [0]),
-        top_k_experts=max([f.top_k for f in ffns] or [0]),
-        arch="nukopel", norm_type="scalar_rmsnorm", act_type="clamped_glu",
+        n_experts=max([getattr(f, "n_experts", 0) for f in ffns] or [0]),
+        top_k_experts=max([getattr(f, "top_k", 0) for f in ffns] or [0]),
+        arch=arch, norm_type=norm_type, act_type=act_type,
         pos_type="rope", layer_specs=list(layer_specs),
         embed_scale=embed_scale, canon_taps=canon_taps,
     )
@@ -446,6 +448,25 @@ def nukopel_spec(name: str, cfg: Dict[str, Any]) -> ModelSpec:
         embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)),
         canon_taps=int((cfg.get("canon") or {}).get("taps", 0)),
         max_seq_len=int(cfg.get("max_seq_len", 32768)),
+    )
+
+
+def pugozen_spec(name: str, cfg: Dict[str, Any],
+                 shapes: Optional[Dict[str, Any]] = None) -> ModelSpec:
+    """Parse a Pugozen config.json dict (parallel-form layers with
+    retention / gated-delta / attention+delta mixers). `shapes` (checkpoint
+    tensor name -> shape) supplies the sizes the config does not state."""
+    from .hybrid import complete_from_shapes, parallel_layer_specs_from_cfg
+
+    layers = parallel_layer_specs_from_cfg(cfg["layers"])
+    if shapes:
+        complete_from_shapes(layers, shapes)
+    return hybrid_spec(
+        name, int(cfg["vocab"]), int(cfg["width"]), layers,
+        eps=float(cfg["norm"]["eps"]),
+        embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)),
+        canon_taps=0, max_seq_len=int(cfg.get("max_seq_len", 32768)),
+        arch="pugozen", norm_type="rmsnorm", act_type="relu2",
     )
 
 
@@ -487,6 +508,12 @@ def spec_from_hf_config(model_path: str, name: Optional[str] = None) -> ModelSpe
     if cfg.get("architecture") == "Nukopel":
         return nukopel_spec(
             name or os.path.basename(os.path.normpath(model_path)), cfg)
+    if cfg.get("architecture") == "Pugozen":
+        from .weights import safetensors_shapes
+
+        return pugozen_spec(
+            name or os.path.basename(os.path.normpath(model_path)), cfg,
+            safetensors_shapes(model_path))
     if cfg.get("model_type") == "gpt2" or "n_embd" in cfg:
         spec = _gpt2(
             name or cfg.get("_name_or_path", os.path.basename(model_path)),

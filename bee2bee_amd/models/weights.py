@@ -39,6 +39,10 @@ class LayerWeights:
         # conv, the latent attention's norm / up-projections, the linear
         # attention's output norm and per-head decay
         "gains", "canon", "kv_norm", "w_uk", "w_uv", "out_norm", "decay",
+        # parallel-form layers: weighted norm, the two fused GEMMs (input
+        # projections incl. the feed-forward's up; mixer outputs + down),
+        # their column layouts, and the mixer parts' small fp32 tensors
+        "norm_w", "w_in", "w_out", "layout", "mix",
     )
 
     def __init__(self) -> None:
@@ -64,6 +68,11 @@ class LayerWeights:
         self.w_uv = None       # [heads, kv_rank, vdim]
         self.out_norm = None   # [heads * vdim] fp32
         self.decay = None      # [heads] fp32
+        self.norm_w = None     # [width] fp32
+        self.w_in = None       # [in_total, width]
+        self.w_out = None      # [width, out_total]
+        self.layout = None     # models/hybrid.py fused_layout(layer)
+        self.mix = None        # {part prefix: SimpleNamespace of tensors}
 
 
 class ModelWeights:
@@ -104,6 +113,8 @@ class ModelWeights:
             if layer_range or expert_range:
                 raise NotImplementedError(
                     "hybrid stacks are not sharded (pipeline/expert ranges)")
+            if s.arch == "pugozen":
+                return self._random_init_pugozen(seed)
             return self._random_init_hybrid(seed)
         lo, hi = layer_range or (0, s.n_layers)
         self.expert_range = expert_range
@@ -201,6 +212,8 @@ class ModelWeights:
             if layer_range or expert_range:
                 raise NotImplementedError(
                     "hybrid stacks are not sharded (pipeline/expert ranges)")
+            if s.arch == "pugozen":
+                return self._load_pugozen(model_path)
             return self._load_nukopel(model_path)
         if s.arch == "gpt2":
             return self._load_gpt2(model_path, layer_range)
@@ -534,6 +547,309 @@ class ModelWeights:
                 lw.w_down = act(get(p + "mlp.shared.down"))
 
 
+    # ------------------------------------------- parallel-form hybrid stacks
+
+    @torch.no_grad()
+    def _load_pugozen(self, model_path: str) -> "ModelWeights":
+        """Pugozen safetensors: 'embed', 'head', 'final.norm' and per layer
+        that owns tensors 'l<i>.norm1', 'l<i>.mix.*' ('.left.*' / '.right.*'
+        for a parallel mixer), 'l<i>.mlp.up|down'. Linear weights [out, in]."""
+        tensors = dict(iter_safetensors(model_path))
+        self._assemble_pugozen(lambda name: tensors.pop(name))
+        return self
+
+    @torch.no_grad()
+    def _random_init_pugozen(self, seed: int) -> "ModelWeights":
+        import zlib
+
+        def get(name: str) -> torch.Tensor:
+            tseed = (seed * 1000003 + zlib.crc32(name.encode())) % (2**31)
+            gen = torch.Generator(device=self.device).manual_seed(tseed)
+            shape, mean, std = self._pugozen_shape(name)
+            t = torch.randn(tuple(shape), generator=gen, dtype=torch.float32,
+                            device=self.device)
+            return (mean + std * t).bfloat16()
+
+        self._assemble_pugozen(get)
+        return self
+
+    def _pugozen_shape(self, name: str):
+        """(shape, init mean, init std) of a checkpoint tensor."""
+        s = self.spec
+        W, V = s.hidden_size, s.vocab_size
+        if name == "embed":
+            return (V, W), 0.0, 1.0 / max(1.0, s.embed_scale)
+        if name == "head":
+            return (V, W), 0.0, W ** -0.5
+        if name == "final.norm":
+            return (W,), 1.0, 0.1
+        head, rest = name.split(".", 1)
+        l = s.layer_specs[int(head[1:])]
+        if rest == "norm1":
+            return (W,), 1.0, 0.1
+        if rest == "mlp.up":
+            return (l.ffn.ff, W), 0.0, W ** -0.5
+        if rest == "mlp.down":
+            return (W, l.ffn.ff), 0.0, l.ffn.ff ** -0.5
+        rest = rest[len("mix."):]
+        m = l.mixer
+        if m.kind == "parallel":
+            side, rest = rest.split(".", 1)
+            m = m.left if side == "left" else m.right
+        H, D, Dv = m.heads, m.dim, m.vdim
+        lin = W ** -0.5
+        if rest == "o":
+            return (W, H * Dv), 0.0, (H * Dv) ** -0.5
+        if m.kind == "retention":
+            return {"q": ((H * D, W), 0.0, lin), "k": ((H * D, W), 0.0, lin),
+                    "v": ((H * Dv, W), 0.0, lin),
+                    "g": ((H * Dv, W), 0.0, lin)}[rest]
+        if m.kind == "sink_attention":
+            G = m.kv_heads
+            return {"q": ((H * D, W), 0.0, lin), "k": ((G * D, W), 0.0, lin),
+                    "q.norm": ((D,), 1.0, 0.1), "k.norm": ((D,), 1.0, 0.1),
+                    "temp": ((H,), 1.0, 0.2), "sink": ((H,), 0.0, 1.0)}[rest]
+        G = m.kv_heads
+        table = {"q": ((G * D, W), 0.0, lin), "k": ((G * D, W), 0.0, lin),
+                 "v": ((H * Dv, W), 0.0, lin),
+                 "q.conv": ((G * D, m.taps), 0.0, 0.4),
+                 "k.conv": ((G * D, m.taps), 0.0, 0.4),
+                 "v.conv": ((H * Dv, m.taps), 0.0, 0.4),
+                 "b": ((H, W), 0.0, lin), "A_log": ((H,), -1.0, 0.5),
+                 "norm": ((Dv,), 1.0, 0.1)}
+        if m.channel_decay:
+            table.update({"a1": ((m.decay_rank, W), 0.0, lin),
+                          "a2": ((H * D, m.decay_rank), 0.0,
+                                 m.decay_rank ** -0.5),
+                          "dt_bias": ((H * D,), 0.0, 0.5)})
+        else:
+            table.update({"a": ((H, W), 0.0, lin), "dt_bias": ((H,), 0.0, 0.5)})
+        if m.gate_rank:
+            table.update({"g1": ((m.gate_rank, W), 0.0, lin),
+                          "g2": ((H * Dv, m.gate_rank), 0.0,
+                                 m.gate_rank ** -0.5)})
+        else:
+            table["g"] = ((H * Dv, W), 0.0, lin)
+        return table[rest]
+
+    def _assemble_pugozen(self, get) -> None:
+        """Engine layout of a parallel-form stack: per layer ONE input GEMM
+        (every projection that reads the normed h, the feed-forward's up
+        included) and ONE output GEMM (mixer output projections and the
+        feed-forward's down side by side along K), segments padded to
+        multiples of 8 (models/hybrid.py fused_layout). A layer with
+        weights_of shares the owning layer's LayerWeights object."""
+        from types import SimpleNamespace
+
+        from .hybrid import fused_layout, mixer_parts
+
+        s = self.spec
+        dev, dt = self.device, self.dtype
+        W = s.hidden_size
+
+        def act(t: torch.Tensor) -> torch.Tensor:
+            return t.to(dev, dt).contiguous()
+
+        def f32(t: torch.Tensor) -> torch.Tensor:
+            return t.to(dev, torch.float32).contiguous()
+
+        self.embed = act(get("embed"))
+        self.lm_head = act(get("head"))
+        self.final_norm = f32(get("final.norm"))
+        for i, l in enumerate(s.layer_specs):
+            if l.weights_of is not None:
+                continue
+            lw, p = self.layers[i], f"l{i}."
+            ins, n_in, outs, n_out = fused_layout(l)
+            lw.layout = (ins, n_in, outs, n_out)
+            lw.norm_w = f32(get(p + "norm1"))
+            w_in = torch.zeros(n_in, W, device=dev, dtype=dt)
+            w_out = torch.zeros(W, n_out, device=dev, dtype=dt)
+
+            def put_in(key: str, t: torch.Tensor) -> None:
+                off, n = ins[key]
+                assert t.shape == (n, W), (key, tuple(t.shape), n)
+                w_in[off : off + n] = t.to(dev, dt)
+
+            lw.mix = {}
+            for pre, m in mixer_parts(l.mixer):
+                q = p + "mix." + pre
+                ns = lw.mix[pre] = SimpleNamespace()
+                if m.kind == "retention":
+                    for n_ in ("q", "k", "v", "g"):
+                        put_in(pre + n_, get(q + n_))
+                    ns.decay = torch.tensor(m.decay, dtype=torch.float32,
+                                            device=dev)
+                elif m.kind == "sink_attention":
+                    put_in(pre + "q", get(q + "q"))
+                    put_in(pre + "k", get(q + "k"))
+                    ns.q_norm = f32(get(q + "q.norm"))
+                    ns.k_norm = f32(get(q + "k.norm"))
+                    ns.temp = f32(get(q + "temp"))
+                    ns.sink = f32(get(q + "sink"))
+                    # score = (q . k) * scale * temp_h, folded into q
+                    ns.q_mult = ns.temp * m.scale
+                else:
+                    put_in(pre + "qkv", torch.cat(
+                        [get(q + "q"), get(q + "k"), get(q + "v")], dim=0))
+                    # checkpoint [channels, taps] -> tap-major [taps, channels]
+                    ns.conv_w = f32(torch.cat(
+                        [get(q + "q.conv"), get(q + "k.conv"),
+                         get(q + "v.conv")], dim=0).t())
+                    put_in(pre + "b", get(q + "b"))
+                    # decay rate exp(A_log), evaluated once in fp32
+                    ns.rate = torch.exp(f32(get(q + "A_log")))
+                    ns.dt_bias = f32(get(q + "dt_bias"))
+                    ns.norm = f32(get(q + "norm"))
+                    if m.channel_decay:
+                        put_in(pre + "a", get(q + "a1"))
+                        ns.a2 = act(get(q + "a2"))
+                    else:
+                        put_in(pre + "a", get(q + "a"))
+                        ns.a2 = None
+                    if m.gate_rank:
+                        put_in(pre + "g", get(q + "g1"))
+                        ns.g2 = act(get(q + "g2"))
+                    else:
+                        put_in(pre + "g", get(q + "g"))
+                        ns.g2 = None
+                off, n = outs[pre + "o"]
+                w_out[:, off : off + n] = get(q + "o").to(dev, dt)
+            if l.ffn is not None:
+                put_in("up", get(p + "mlp.up"))
+                off, n = outs["down"]
+                w_out[:, off : off + n] = get(p + "mlp.down").to(dev, dt)
+            lw.w_in, lw.w_out = w_in, w_out
+        for i, l in enumerate(s.layer_specs):
+            if l.weights_of is not None:
+                self.layers[i] = self.layers[l.weights_of]
+
+
+def safetensors_shapes(model_path: str) -> Dict[str, Tuple[int, ...]]:
+    """Tensor name -> shape from the shards' headers (8-byte little-endian
+    length, then that many bytes of JSON); no tensor data is read."""
+    import struct
+
+    out: Dict[str, Tuple[int, ...]] = {}
+    for shard in sorted(glob.glob(os.path.join(model_path, "*.safetensors"))):
+        with open(shard, "rb") as f:
+            (n,) = struct.unpack("<Q", f.read(8))
+            header = json.loads(f.read(n))
+        for name, meta in header.items():
+            if name != "__metadata__":
+                out[name] = tuple(meta["shape"])
+    return out
+
+
+def pugozen_config(spec: ModelSpec) -> Dict:
+    """The config.json dict of a Pugozen spec (inverse of pugozen_spec)."""
+    def rot(m):
+        return {"base": m.rope_base, "dims": m.rope_dims}
+
+    def delta(m):
+        return {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim,
+                "vdim": m.vdim, "conv": m.taps}
+
+    layers = []
+    for l in spec.layer_specs:
+        m = l.mixer
+        if m.kind == "retention":
+            mixer = {"heads": m.heads, "dim": m.dim, "vdim": m.vdim,
+                     "decay": list(m.decay), "rot": rot(m)}
+        elif m.kind == "delta":
+            mixer = delta(m)
+        else:
+            a = m.left
+            mixer = {"left": {"heads": a.heads, "kv_heads": a.kv_heads,
+                              "dim": a.dim, "vdim": a.vdim, "scale": a.scale,
+                              "rot": rot(a)},
+                     "right": delta(m.right), "left_scale": m.left_scale,
+                     "right_scale": m.right_scale}
+        entry = {"type": m.kind, "mixer": mixer,
+                 "mlp": ({"kind": "dense", "ff": l.ffn.ff}
+                         if l.ffn is not None else None)}
+        if l.weights_of is not None:
+            entry["weights_of"] = l.weights_of
+        layers.append(entry)
+    return {"architecture": "Pugozen", "vocab": spec.vocab_size,
+            "width": spec.hidden_size,
+            "embedding": {"scale": spec.embed_scale},
+            "norm": {"eps": spec.rms_eps}, "max_seq_len": spec.max_seq_len,
+            "layers": layers}
+
+
+def _save_pugozen(weights: "ModelWeights", out_dir: str, tensors, cpu) -> None:
+    """Pugozen-format shard + config: the two fused matrices split back
+    into the checkpoint's tensors (bf16, [out, in])."""
+    from safetensors.torch import save_file
+
+    from .hybrid import mixer_parts
+
+    s = weights.spec
+
+    def put(name: str, t: torch.Tensor) -> None:
+        tensors[name] = cpu(t).to(torch.bfloat16).contiguous()
+
+    put("embed", weights.embed)
+    put("head", weights.lm_head)
+    put("final.norm", weights.final_norm)
+    for i, l in enumerate(s.layer_specs):
+        if l.weights_of is not None:
+            continue
+        lw, p = weights.layers[i], f"l{i}."
+        ins, _, outs, _ = lw.layout
+
+        def rows(key: str) -> torch.Tensor:
+            off, n = ins[key]
+            return lw.w_in[off : off + n]
+
+        put(p + "norm1", lw.norm_w)
+        for pre, m in mixer_parts(l.mixer):
+            q, ns = p + "mix." + pre, lw.mix[pre]
+            if m.kind == "retention":
+                for n_ in ("q", "k", "v", "g"):
+                    put(q + n_, rows(pre + n_))
+            elif m.kind == "sink_attention":
+                put(q + "q", rows(pre + "q"))
+                put(q + "k", rows(pre + "k"))
+                put(q + "q.norm", ns.q_norm)
+                put(q + "k.norm", ns.k_norm)
+                put(q + "temp", ns.temp)
+                put(q + "sink", ns.sink)
+            else:
+                nq = m.kv_heads * m.dim
+                parts = torch.split(rows(pre + "qkv"),
+                                    [nq, nq, m.heads * m.vdim], dim=0)
+                convs = torch.split(ns.conv_w.t(), [nq, nq, m.heads * m.vdim],
+                                    dim=0)
+                for n_, t, c in zip("qkv", parts, convs):
+                    put(q + n_, t)
+                    put(q + n_ + ".conv", c)
+                put(q + "b", rows(pre + "b"))
+                put(q + "A_log", torch.log(ns.rate))
+                put(q + "dt_bias", ns.dt_bias)
+                put(q + "norm", ns.norm)
+                if m.channel_decay:
+                    put(q + "a1", rows(pre + "a"))
+                    put(q + "a2", ns.a2)
+                else:
+                    put(q + "a", rows(pre + "a"))
+                if m.gate_rank:
+                    put(q + "g1", rows(pre + "g"))
+                    put(q + "g2", ns.g2)
+                else:
+                    put(q + "g", rows(pre + "g"))
+            off, n = outs[pre + "o"]
+            put(q + "o", lw.w_out[:, off : off + n])
+        if l.ffn is not None:
+            put(p + "mlp.up", rows("up"))
+            off, n = outs["down"]
+            put(p + "mlp.down", lw.w_out[:, off : off + n])
+    save_file(tensors, os.path.join(out_dir, "model.safetensors"))
+    with open(os.path.join(out_dir, "config.json"), "w") as fh:
+        json.dump(pugozen_config(s), fh, indent=1)
+
+
 def _save_gpt2(weights: "ModelWeights", out_dir: str, tensors, cpu) -> None:
     """GPT-2-format shard + config (Conv1D tensors re-transposed)."""
     from safetensors.torch import save_file
@@ -698,7 +1014,10 @@ def save_hf(weights: ModelWeights, out_dir: str) -> None:
         _save_gpt2(weights, out_dir, tensors, cpu)
         return
     if s.is_hybrid:
-        _save_nukopel(weights, out_dir, tensors, cpu)
+        if s.arch == "pugozen":
+            _save_pugozen(weights, out_dir, tensors, cpu)
+        else:
+            _save_nukopel(weights, out_dir, tensors, cpu)
         return
 
     if weights.embed is not None:

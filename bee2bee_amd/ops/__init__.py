@@ -316,3 +316,103 @@ def clamped_glu(gate_up, limit: float, alpha: float):
     if _use_hip(gate_up):
         return require_hip().clamped_glu(gate_up, float(limit), float(alpha))
     return reference.clamped_glu(gate_up, limit, alpha)
+
+
+# ---------------------------------------------- parallel-form hybrid stacks
+# (ops/reference.py documents shapes). Ops with an `out` argument write a
+# strided column slice of a wider activation buffer in place.
+
+rope_tables_f64 = reference.rope_tables_f64
+
+
+def rmsnorm_f32(x, w, eps: float, out_dtype):
+    if _use_hip(x):
+        return require_hip().add_rmsnorm_f32(x, None, w, eps, out_dtype, False)
+    return reference.rmsnorm_f32(x, w, eps, out_dtype)
+
+
+def add_rmsnorm_f32(resid, y, w, eps: float, out_dtype):
+    """resid(fp32) += y in place; -> unit(resid) * w (None when w is None)."""
+    if _use_hip(resid):
+        return require_hip().add_rmsnorm_f32(resid, y, w, eps, out_dtype, True)
+    return reference.add_rmsnorm_f32(resid, y, w, eps, out_dtype)
+
+
+def relu2(x, out) -> None:
+    if _use_hip(x):
+        require_hip().relu2(x, out)
+        return
+    reference.relu2(x, out)
+
+
+def qk_norm_rope_store(q, k, q_norm, k_norm, eps: float, rope_dims: int,
+                       positions, cos, sin, q_mult, k_cache, v_cache,
+                       slot_mapping) -> None:
+    if _use_hip(q):
+        require_hip().qk_norm_rope_store(q, k, q_norm, k_norm, eps, rope_dims,
+                                         positions, cos, sin, q_mult, k_cache,
+                                         v_cache, slot_mapping)
+        return
+    reference.qk_norm_rope_store(q, k, q_norm, k_norm, eps, rope_dims,
+                                 positions, cos, sin, q_mult, k_cache,
+                                 v_cache, slot_mapping)
+
+
+def sink_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
+              cu_seqlens, sink, window: int, out, out_scale: float,
+              max_qlen: int = 0) -> None:
+    if _use_hip(q):
+        require_hip().sink_attn(q, k_cache, v_cache, block_table, positions,
+                                seq_idx, cu_seqlens, sink, window, out,
+                                float(out_scale), max_qlen)
+        return
+    reference.sink_attn(q, k_cache, v_cache, block_table, positions, seq_idx,
+                        cu_seqlens, sink, window, out, out_scale)
+
+
+def short_conv(x, w, state, state_slots, cu_seqlens, seq_idx, positions,
+               silu: bool = True):
+    if _use_hip(x):
+        return require_hip().short_conv(x, w, state, state_slots, cu_seqlens,
+                                        seq_idx, positions, silu)
+    return reference.short_conv(x, w, state, state_slots, cu_seqlens, seq_idx,
+                                positions, silu)
+
+
+def delta_gates(qk, n_qk_heads: int, dim: int, b, a, dt_bias, rate,
+                channel_decay: bool):
+    if _use_hip(qk):
+        return tuple(require_hip().delta_gates(qk, n_qk_heads, dim, b, a,
+                                               dt_bias, rate, channel_decay))
+    return reference.delta_gates(qk, n_qk_heads, dim, b, a, dt_bias, rate,
+                                 channel_decay)
+
+
+def delta_rule(q, k, v, beta, g, state, state_slots, cu_seqlens, positions):
+    if _use_hip(q):
+        return require_hip().delta_rule(q, k, v, beta, g, state, state_slots,
+                                        cu_seqlens, positions)
+    return reference.delta_rule(q, k, v, beta, g, state, state_slots,
+                                cu_seqlens, positions)
+
+
+def head_gated_norm(o, w, gate, gate_act: str, eps: float, out,
+                    out_scale: float) -> None:
+    if _use_hip(o):
+        require_hip().head_gated_norm(o, w, gate, gate_act == "sigmoid", eps,
+                                      out, float(out_scale))
+        return
+    reference.head_gated_norm(o, w, gate, gate_act, eps, out, out_scale)
+
+
+def retention_attn(q, k, v, decay, rope_dims: int, cos, sin, k_scale: float,
+                   state, state_slots, cu_seqlens, positions,
+                   max_qlen: int = 0):
+    if _use_hip(q):
+        return require_hip().retention_attn(q, k, v, decay, rope_dims, cos,
+                                            sin, float(k_scale), state,
+                                            state_slots, cu_seqlens,
+                                            positions, max_qlen)
+    return reference.retention_attn(q, k, v, decay, rope_dims, cos, sin,
+                                    k_scale, state, state_slots, cu_seqlens,
+                                    positions)

@@ -519,3 +519,299 @@ def clamped_glu(gate_up: torch.Tensor, limit: float,
     g = g.clamp(max=limit)
     u = u.clamp(min=-limit, max=limit)
     return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gate_up.dtype)
+
+
+# ---------------------------------------------- parallel-form hybrid stacks
+#
+# Mechanisms of stacks whose layers are x += mixer(h) + ffn(h) with
+# h = unit(x) * w: weighted fp32 norms, grouped-query attention with a sink
+# logit, retention (decayed linear attention on rotated q/k), the gated
+# delta rule with its short convolution, per-head gated output norms.
+# Several ops write into a column slice of a wider activation buffer (`out`
+# is a strided [T, n] view), so one GEMM can consume all of them.
+
+
+def rope_tables_f64(max_len: int, dims: int, base: float, device
+                    ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """cos/sin [max_len, dims/2] of angle p * base^(-2i/dims), evaluated in
+    float64 and rounded once to fp32."""
+    i = torch.arange(0, dims, 2, dtype=torch.float64)
+    inv = torch.pow(torch.tensor(float(base), dtype=torch.float64), -i / dims)
+    ang = torch.outer(torch.arange(max_len, dtype=torch.float64), inv)
+    return (ang.cos().to(device, torch.float32),
+            ang.sin().to(device, torch.float32))
+
+
+def rmsnorm_f32(x: torch.Tensor, w: torch.Tensor, eps: float,
+                out_dtype: torch.dtype) -> torch.Tensor:
+    """fp32 rows -> unit(x) * w in out_dtype."""
+    xf = x.float()
+    r = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    return (xf * r * w.float()).to(out_dtype)
+
+
+def add_rmsnorm_f32(resid: torch.Tensor, y: torch.Tensor,
+                    w: Optional[torch.Tensor], eps: float,
+                    out_dtype: torch.dtype) -> Optional[torch.Tensor]:
+    """resid (fp32, in place) += y; returns unit(resid) * w (None if w is)."""
+    resid.add_(y.float())
+    if w is None:
+        return None
+    return rmsnorm_f32(resid, w, eps, out_dtype)
+
+
+def relu2(x: torch.Tensor, out: torch.Tensor) -> None:
+    """out <- relu(x)^2 (both may be strided column slices)."""
+    z = torch.relu(x.float())
+    out.copy_((z * z).to(out.dtype))
+
+
+def qk_norm_rope_store(q: torch.Tensor, k: torch.Tensor, q_norm: torch.Tensor,
+                       k_norm: torch.Tensor, eps: float, rope_dims: int,
+                       positions: torch.Tensor, cos, sin,
+                       q_mult: torch.Tensor, k_cache: torch.Tensor,
+                       v_cache: torch.Tensor,
+                       slot_mapping: torch.Tensor) -> None:
+    """q [T, H, D] (view, rewritten in place): rotate(unit(q) * q_norm) *
+    q_mult[h]. k [T, G, D] (view, left as is): rotate(unit(k) * k_norm) goes
+    to k_cache, k itself (the value) to v_cache, both
+    [n_blocks, G, block, D] at slot_mapping."""
+    T, G, D = k.shape
+    bs = k_cache.shape[2]
+    qf, kf = q.float(), k.float()
+    qn = qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + eps) * q_norm
+    kn = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps) * k_norm
+    if rope_dims:
+        p = positions.long()
+        c, s = cos[p][:, None], sin[p][:, None]
+        qn = _rot_half(qn, c, s, rope_dims)
+        kn = _rot_half(kn, c, s, rope_dims)
+    q.copy_((qn * q_mult.float()[None, :, None]).to(q.dtype))
+    slot = slot_mapping.long()
+    blk, off = slot // bs, slot % bs
+    k_cache[blk, :, off] = kn.to(k_cache.dtype)
+    v_cache[blk, :, off] = k.to(v_cache.dtype)
+
+
+def sink_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+              block_table: torch.Tensor, positions: torch.Tensor,
+              seq_idx: torch.Tensor, cu_seqlens: torch.Tensor,
+              sink: Optional[torch.Tensor], window: int, out: torch.Tensor,
+              out_scale: float) -> None:
+    """Causal grouped-query attention over the pages; scores are q . k (all
+    multipliers are already in q). Row t at position p of chunk b sees
+    cached positions j <= p (and j > p - window when window > 0). The
+    softmax denominator also holds exp(sink[h]) when sink is given.
+    out [T, H * Dv] (strided view) <- attention * out_scale."""
+    T, H, D = q.shape
+    G, bs, Dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    rep = H // G
+    cu = cu_seqlens.tolist()
+    res = torch.zeros(T, H, Dv, dtype=torch.float32, device=q.device)
+    for b in range(len(cu) - 1):
+        lo, hi = cu[b], cu[b + 1]
+        if hi == lo:
+            continue
+        pos = positions[lo:hi].long()
+        k_lo = max(0, int(pos.min()) - window + 1) if window > 0 else 0
+        k_hi = int(pos.max()) + 1
+        kpos = torch.arange(k_lo, k_hi, device=q.device)
+        blk = block_table[b].long()[kpos // bs]
+        keys = k_cache[blk, :, kpos % bs].float()          # [S, G, D]
+        vals = v_cache[blk, :, kpos % bs].float()          # [S, G, Dv]
+        qb = q[lo:hi].float().view(hi - lo, G, rep, D)
+        s = torch.einsum("tgrd,sgd->grts", qb, keys)
+        d = pos[:, None] - kpos[None, :]
+        dead = d < 0
+        if window > 0:
+            dead = dead | (d >= window)
+        s.masked_fill_(dead[None, None], float("-inf"))
+        m = s.max(-1, keepdim=True).values
+        if sink is not None:
+            sk = sink.float().view(G, rep, 1, 1)
+            m = torch.maximum(m, sk)
+        e = torch.exp(s - m)
+        den = e.sum(-1, keepdim=True)
+        if sink is not None:
+            den = den + torch.exp(sk - m)
+        o = torch.einsum("grts,sgv->tgrv", e / den, vals)
+        res[lo:hi] = o.reshape(hi - lo, H, Dv)
+    out.copy_((res.view(T, H * Dv) * out_scale).to(out.dtype))
+
+
+def short_conv(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor,
+               state_slots: torch.Tensor, cu_seqlens: torch.Tensor,
+               seq_idx: torch.Tensor, positions: torch.Tensor,
+               silu: bool = True) -> torch.Tensor:
+    """Causal per-channel conv over time (+ silu) -> fp32 [T, C]. x [T, C]
+    may be a strided column slice; w [taps, C] tap-major (last row is the
+    current token's); state [n_slots, taps-1, C] holds each sequence's last
+    taps-1 inputs and is advanced in place. Rows before position 0 are zero
+    by select."""
+    T, C = x.shape
+    K = w.shape[0] - 1
+    wf, xf = w.float(), x.float()
+    out = xf * wf[K]
+    if K > 0:
+        sidx = seq_idx.long()
+        rows = torch.arange(T, device=x.device)
+        cu = cu_seqlens.long()
+        local = rows - cu[sidx]
+        slots = state_slots.long()[sidx]
+        pos = positions.long()
+        for d in range(1, K + 1):
+            src = local - d
+            val = torch.where((src >= 0)[:, None], xf[(rows - d).clamp(min=0)],
+                              state[slots, (K + src).clamp(0, K - 1)].float())
+            val = torch.where((pos - d >= 0)[:, None], val,
+                              torch.zeros_like(val))
+            out += wf[K - d] * val
+        lens = cu[1:] - cu[:-1]
+        kk = torch.arange(K, device=x.device)
+        src = lens[:, None] - K + kk[None, :]                    # [B, K]
+        st = state_slots.long()
+        new = torch.where(
+            (src >= 0)[..., None],
+            x[(cu[:-1, None] + src).clamp(0, T - 1)].to(state.dtype),
+            state[st[:, None], (K + src).clamp(0, K - 1)])
+        live = lens > 0
+        state[st[live]] = new[live]
+    if silu:
+        out = torch.nn.functional.silu(out)
+    return out
+
+
+def delta_gates(qk: torch.Tensor, n_qk_heads: int, dim: int, b: torch.Tensor,
+                a: torch.Tensor, dt_bias: torch.Tensor, rate: torch.Tensor,
+                channel_decay: bool):
+    """The fp32 inputs of a delta-rule recurrence besides v.
+    qk fp32 [T, >= 2*n_qk_heads*dim] (conv output; q heads then k heads):
+    made unit vectors per head IN PLACE, x / sqrt(sum x^2 + 1e-6), q also
+    times dim^-1/2. Returns beta = sigmoid(b) [T, H] and the decay
+    g = exp(-rate_h * softplus(a + dt_bias)), [T, H] or (channel_decay)
+    [T, H * dim]."""
+    T = qk.shape[0]
+    n = n_qk_heads * dim
+    for j, mult in ((0, dim ** -0.5), (1, 1.0)):
+        part = qk[:, j * n : (j + 1) * n].view(T, n_qk_heads, dim)
+        part.mul_(torch.rsqrt(part.pow(2).sum(-1, keepdim=True) + 1e-6) * mult)
+    beta = torch.sigmoid(b.float())
+    sp = torch.nn.functional.softplus(a.float() + dt_bias.float())
+    H = rate.numel()
+    if channel_decay:
+        g = torch.exp(-rate.float().view(1, H, 1) * sp.view(T, H, dim))
+        g = g.reshape(T, H * dim)
+    else:
+        g = torch.exp(-rate.float() * sp)
+    return beta.contiguous(), g.contiguous()
+
+
+def delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+               beta: torch.Tensor, g: torch.Tensor, state: torch.Tensor,
+               state_slots: torch.Tensor, cu_seqlens: torch.Tensor,
+               positions: torch.Tensor) -> torch.Tensor:
+    """Gated delta rule, fp32, token by token per sequence chunk.
+    q, k [T, G, D] and v [T, H, Dv] fp32 (strided views allowed; value head
+    h uses q/k head h // (H/G)); beta [T, H]; g [T, H] or [T, H*D] (fade of
+    the memory rows that belong to key channels); state [n_slots, H, D, Dv]
+    fp32 (the memory M), read unless the chunk starts at position 0,
+    advanced in place. Per token, in this order:
+      M <- g * M;  delta = beta (v - M^T k);  M <- M + k delta^T;  y = M^T q
+    Returns y fp32 [T, H, Dv]."""
+    T, G, D = q.shape
+    H, Dv = v.shape[1], v.shape[2]
+    rep = H // G
+    out = torch.empty(T, H, Dv, dtype=torch.float32, device=q.device)
+    per_channel = g.shape[1] != H
+    cu = cu_seqlens.tolist()
+    for b in range(len(cu) - 1):
+        lo, hi = cu[b], cu[b + 1]
+        if hi == lo:
+            continue
+        slot = int(state_slots[b])
+        if int(positions[lo]) == 0:
+            S = torch.zeros(H, D, Dv, dtype=torch.float32, device=q.device)
+        else:
+            S = state[slot].clone()
+        qq = q[lo:hi].float().repeat_interleave(rep, dim=1)
+        kk = k[lo:hi].float().repeat_interleave(rep, dim=1)
+        vv = v[lo:hi].float()
+        gg = g[lo:hi].view(hi - lo, H, D, 1) if per_channel \
+            else g[lo:hi].view(hi - lo, H, 1, 1)
+        bb = beta[lo:hi]
+        for t in range(hi - lo):
+            S = S * gg[t]
+            u = bb[t][:, None] * (vv[t] - torch.einsum("hdv,hd->hv", S, kk[t]))
+            S = S + kk[t][:, :, None] * u[:, None, :]
+            out[lo + t] = torch.einsum("hdv,hd->hv", S, qq[t])
+        state[slot] = S
+    return out
+
+
+def head_gated_norm(o: torch.Tensor, w: Optional[torch.Tensor],
+                    gate: torch.Tensor, gate_act: str, eps: float,
+                    out: torch.Tensor, out_scale: float) -> None:
+    """o fp32 [T, H, Dv]: per head unit(o) [* w (Dv, shared by heads)] *
+    act(gate) * out_scale -> out [T, H*Dv] (strided view, activation dtype).
+    gate [T, H*Dv] raw (strided view); act is "silu" or "sigmoid"."""
+    T, H, Dv = o.shape
+    of = o.float()
+    y = of * torch.rsqrt(of.pow(2).mean(-1, keepdim=True) + eps)
+    if w is not None:
+        y = y * w.float()
+    gf = gate.float().view(T, H, Dv)
+    ga = torch.sigmoid(gf) if gate_act == "sigmoid" else \
+        torch.nn.functional.silu(gf)
+    out.copy_((y * ga * out_scale).reshape(T, H * Dv).to(out.dtype))
+
+
+def retention_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                   decay: torch.Tensor, rope_dims: int, cos, sin,
+                   k_scale: float, state: torch.Tensor,
+                   state_slots: torch.Tensor, cu_seqlens: torch.Tensor,
+                   positions: torch.Tensor) -> torch.Tensor:
+    """Decayed linear attention on rotated queries/keys, fp32 throughout:
+    q, k [T, H, D] raw projections are rotated by position (first rope_dims
+    coordinates, pairs (i, i + rope_dims/2)), k times k_scale; per token
+    M <- lam_h M + k v^T, y = M^T q. Chunked evaluation (intra-chunk decay
+    matrix + carried state). Returns y fp32 [T, H*Dv]."""
+    T, H, D = q.shape
+    Dv = v.shape[-1]
+    qf, kf = q.float(), k.float()
+    if rope_dims:
+        p = positions.long()
+        c, s = cos[p][:, None], sin[p][:, None]
+        qf = _rot_half(qf, c, s, rope_dims)
+        kf = _rot_half(kf, c, s, rope_dims)
+    kf = kf * k_scale
+    out = torch.empty(T, H, Dv, dtype=torch.float32, device=q.device)
+    cu = cu_seqlens.tolist()
+    log_lam = torch.log(decay.float())
+    for b in range(len(cu) - 1):
+        lo, hi = cu[b], cu[b + 1]
+        if hi == lo:
+            continue
+        slot = int(state_slots[b])
+        if int(positions[lo]) == 0:
+            S = torch.zeros(H, D, Dv, dtype=torch.float32, device=q.device)
+        else:
+            S = state[slot].clone()
+        for c0 in range(lo, hi, LIGHTNING_CHUNK):
+            c1 = min(hi, c0 + LIGHTNING_CHUNK)
+            n = c1 - c0
+            qc = qf[c0:c1].transpose(0, 1)                  # [H, n, D]
+            kc = kf[c0:c1].transpose(0, 1)
+            vc = v[c0:c1].float().transpose(0, 1)           # [H, n, Dv]
+            i = torch.arange(n, device=q.device, dtype=torch.float32)
+            diff = i[:, None] - i[None, :]
+            M = torch.exp(log_lam[:, None, None] * diff.clamp(min=0))
+            M = M * (diff >= 0)
+            o = torch.bmm(torch.bmm(qc, kc.transpose(1, 2)) * M, vc)
+            carry = torch.exp(log_lam[:, None] * (i + 1.0))
+            o += torch.bmm(qc, S) * carry[..., None]
+            out[c0:c1] = o.transpose(0, 1)
+            tail = torch.exp(log_lam[:, None] * (n - 1.0 - i))
+            S = S * torch.exp(log_lam * n)[:, None, None] + torch.bmm(
+                (kc * tail[..., None]).transpose(1, 2), vc)
+        state[slot] = S
+    return out.view(T, H * Dv)
