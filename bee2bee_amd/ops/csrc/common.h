@@ -85,6 +85,16 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 #define DEV_INLINE __device__ __forceinline__
 
+// LDS hand-over inside ONE wave (no workgroup barrier): a wave's LDS
+// operations execute in order, so earlier writes of any lane are seen by
+// later reads of any lane; the fences keep the compiler from moving them.
+#define WAVE_LDS_SYNC()                                                       \
+    do {                                                                      \
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                \
+        __builtin_amdgcn_wave_barrier();                                      \
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");                \
+    } while (0)
+
 // Debug-assert build (BEE2BEE_DEBUG_KERNELS=1 at build time -> hipcc gets
 // -DBEE2BEE_DEBUG): bounds/invariant checks compile into the kernels and
 // trap with file:line on violation. The release build compiles them away

@@ -195,18 +195,21 @@ __global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ y,
 }
 
 // ------------------------------------------------------- input convolution
-// out[t] = h[t] + sum_d w[K-d][c] * h[t-d], d = 0..K (K = taps-1). Rows
-// before the chunk come from the sequence's state (its last K inputs), rows
-// before position 0 are zero.
-template <typename T, int VEC>
-__global__ void canon_conv_kernel(const T* __restrict__ h,
+// out[t] = [h[t] +] sum_d w[K-d][c] * h[t-d], d = 0..K (K = taps-1), then
+// silu when SILU. RES adds the input itself (the whole-width conv of the
+// sandwich layers); the short conv of a delta mixer is plain and activated.
+// h may be a column slice of a wider buffer (row stride hs); out is
+// contiguous [T, C] of type OT. Rows before the chunk come from the
+// sequence's state (its last K inputs), rows before position 0 are zero.
+template <typename T, typename OT, int VEC, bool RES, bool SILU>
+__global__ void canon_conv_kernel(const T* __restrict__ h, long hs,
                                   const float* __restrict__ w,   // [K+1, C]
                                   const T* __restrict__ state,   // [S, K, C]
                                   const int* __restrict__ state_slots,
                                   const int* __restrict__ cu,
                                   const int* __restrict__ seq_idx,
                                   const int* __restrict__ positions,
-                                  T* __restrict__ out, int C, int K) {
+                                  OT* __restrict__ out, int C, int K) {
     const long t = blockIdx.x;
     const int c = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
     if (c >= C) return;
@@ -215,28 +218,33 @@ __global__ void canon_conv_kernel(const T* __restrict__ h,
     const int pos = positions[t];
     const long slot = state_slots[b];
     float acc[VEC], v[VEC], wv[VEC];
-    ldv<T, VEC>(h + t * C + c, v);
+    ldv<T, VEC>(h + t * hs + c, v);
     ldv<float, VEC>(w + (long)K * C + c, wv);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) acc[j] = v[j] * (1.f + wv[j]);
+    for (int j = 0; j < VEC; ++j)
+        acc[j] = v[j] * (RES ? 1.f + wv[j] : wv[j]);
     for (int d = 1; d <= K; ++d) {
         if (pos - d < 0) break;
         const int src = local - d;
         if (src >= 0)
-            ldv<T, VEC>(h + (t - d) * C + c, v);
+            ldv<T, VEC>(h + (t - d) * hs + c, v);
         else
             ldv<T, VEC>(state + (slot * K + (K + src)) * C + c, v);
         ldv<float, VEC>(w + (long)(K - d) * C + c, wv);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) acc[j] += wv[j] * v[j];
     }
-    stv<T, VEC>(out + t * C + c, acc);
+    if (SILU) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] = acc[j] / (1.f + expf(-acc[j]));
+    }
+    stv<OT, VEC>(out + t * C + c, acc);
 }
 
 // state <- the sequence's last K inputs after this chunk (thread per
 // channel reads all K old rows before it writes any).
 template <typename T>
-__global__ void canon_state_kernel(const T* __restrict__ h,
+__global__ void canon_state_kernel(const T* __restrict__ h, long hs,
                                    T* __restrict__ state,
                                    const int* __restrict__ state_slots,
                                    const int* __restrict__ cu, int C, int K) {
@@ -250,7 +258,7 @@ __global__ void canon_state_kernel(const T* __restrict__ h,
     for (int k = 0; k < K; ++k) keep[k] = st[(long)k * C];
     for (int k = 0; k < K; ++k) {
         const int src = L - K + k;
-        st[(long)k * C] = src >= 0 ? h[(long)(lo + src) * C + c]
+        st[(long)k * C] = src >= 0 ? h[(long)(lo + src) * hs + c]
                                    : keep[K + src];
     }
 }
@@ -307,6 +315,203 @@ __global__ void latent_rope_store_kernel(
 }
 
 }  // namespace
+
+// ------------------------------------------- weighted fp32-residual norm
+// resid (fp32) += y when y is given; out = unit(resid) * w when out is.
+// One workgroup per row, the row held in LDS between the passes.
+template <typename YT, typename OT, int VEC>
+__global__ void add_rmsnorm_w_kernel(float* __restrict__ resid,
+                                     const YT* __restrict__ y,
+                                     const float* __restrict__ w,
+                                     OT* __restrict__ out, int W, float eps) {
+    extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+    float* row = reinterpret_cast<float*>(smem_raw);
+    __shared__ float red[16];
+    const long t = blockIdx.x;
+    float* rr = resid + t * (long)W;
+    const YT* yr = y ? y + t * (long)W : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x * VEC; i < W; i += blockDim.x * VEC) {
+        float v[VEC];
+        ldv<float, VEC>(rr + i, v);
+        if (yr) {
+            float a[VEC];
+            ldv<YT, VEC>(yr + i, a);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] += a[j];
+            stv<float, VEC>(rr + i, v);
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            row[i + j] = v[j];
+            ss += v[j] * v[j];
+        }
+    }
+    if (!out) return;
+    const float r = 1.f / sqrtf(block_sum(ss, red) / (float)W + eps);
+    OT* orow = out + t * (long)W;
+    for (int i = threadIdx.x * VEC; i < W; i += blockDim.x * VEC) {
+        float v[VEC], wv[VEC];
+        ldv<float, VEC>(w + i, wv);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = row[i + j] * r * wv[j];
+        stv<OT, VEC>(orow + i, v);
+    }
+}
+
+// --------------------------------------------------------------- relu^2
+// out[r, c] = max(x[r, c], 0)^2 over column slices (row strides xs, os)
+template <typename T, int VEC>
+__global__ void relu2_kernel(const T* __restrict__ x, long xs,
+                             T* __restrict__ out, long os, long rows, int n) {
+    const int per = n / VEC;
+    const long total = rows * per;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const long r = idx / per;
+        const int c = (int)(idx - r * per) * VEC;
+        float v[VEC];
+        ldv<T, VEC>(x + r * xs + c, v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            const float z = fmaxf(v[j], 0.f);
+            v[j] = z * z;
+        }
+        stv<T, VEC>(out + r * os + c, v);
+    }
+}
+
+// ------------------------------------------------- per-head gated norm
+// Wave per (token, head): y = unit(o_head) [* w] * act(gate) * out_scale,
+// act = silu or sigmoid. o fp32 [T, H, Dv]; gate and out are column slices.
+template <typename T>
+__global__ void head_gated_norm_kernel(const float* __restrict__ o,
+                                       const float* __restrict__ w,
+                                       const T* __restrict__ gate, long gs,
+                                       T* __restrict__ out, long os, long rows,
+                                       int H, int Dv, float eps, int sigmoid,
+                                       float out_scale) {
+    const long row = (long)blockIdx.x * (blockDim.x / WAVE) +
+                     threadIdx.x / WAVE;       // (token, head)
+    if (row >= rows) return;
+    const int lane = threadIdx.x % WAVE;
+    const long t = row / H;
+    const int h = (int)(row - t * H);
+    const float* orow = o + row * Dv;
+    float ss = 0.f;
+    for (int i = lane; i < Dv; i += WAVE) ss += orow[i] * orow[i];
+    const float r = out_scale / sqrtf(wave_sum(ss) / (float)Dv + eps);
+    const T* gr = gate + t * gs + (long)h * Dv;
+    T* yr = out + t * os + (long)h * Dv;
+    for (int i = lane; i < Dv; i += WAVE) {
+        const float g = ldf(gr + i);
+        const float sg = 1.f / (1.f + expf(-g));
+        float v = orow[i] * r * (sigmoid ? sg : g * sg);
+        if (w) v *= w[i];
+        stf(yr + i, v);
+    }
+}
+
+// ------------------------------------------------ delta-rule gate inputs
+// Workgroup per token. (1) the 2*NQ q/k heads of the fp32 conv output are
+// made unit vectors in place, x / sqrt(sum x^2 + 1e-6), q also times
+// D^-1/2; (2) beta = sigmoid(b); (3) decay g = exp(-rate_h *
+// softplus(a + dt_bias)), one per head or one per head and key channel.
+template <typename T>
+__global__ void delta_gates_kernel(float* __restrict__ qk, long qs, int NQ,
+                                   int D, const T* __restrict__ b, long bs,
+                                   const T* __restrict__ a, long as,
+                                   const float* __restrict__ dt_bias,
+                                   const float* __restrict__ rate,
+                                   float* __restrict__ beta,
+                                   float* __restrict__ g, int H, int per_head) {
+    const long t = blockIdx.x;
+    const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int nw = blockDim.x / WAVE;
+    float* row = qk + t * qs;
+    const float qmul = 1.f / sqrtf((float)D);
+    for (int hh = wid; hh < 2 * NQ; hh += nw) {
+        float* v = row + (long)hh * D;
+        float ss = 0.f;
+        for (int i = lane; i < D; i += WAVE) ss += v[i] * v[i];
+        const float r = (hh < NQ ? qmul : 1.f) / sqrtf(wave_sum(ss) + 1e-6f);
+        for (int i = lane; i < D; i += WAVE) v[i] *= r;
+    }
+    for (int h = threadIdx.x; h < H; h += blockDim.x)
+        beta[t * H + h] = 1.f / (1.f + expf(-ldf(b + t * bs + h)));
+    const int n = H * per_head;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const float z = ldf(a + t * as + i) + dt_bias[i];
+        const float sp = z > 20.f ? z : log1pf(expf(z));
+        g[t * n + i] = expf(-rate[i / per_head] * sp);
+    }
+}
+
+// ------------------------------------- query/key norm, rotation, page store
+// Workgroup per token, a wave per head in turn (H query heads, then G key
+// heads). Query head: q <- rotate(unit(q) * wq) * q_mult[h] in place. Key
+// head: rotate(unit(k) * wk) -> k_cache, k as projected -> v_cache (pages
+// [n_blocks, G, bs, D]). Rotation pairs dim i with i + dims/2 over the
+// first `dims` coordinates; cos/sin fp32 tables [max_pos, dims/2].
+constexpr int QKN_MAXD = 512;
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_store_kernel(T* __restrict__ q, long q_tok, int H,
+                          const T* __restrict__ k, long k_tok, int G, int D,
+                          const float* __restrict__ wq,
+                          const float* __restrict__ wk, float eps, int dims,
+                          const int* __restrict__ positions,
+                          const float* __restrict__ cos_t,
+                          const float* __restrict__ sin_t,
+                          const float* __restrict__ q_mult,
+                          T* __restrict__ k_cache, T* __restrict__ v_cache,
+                          int bs, const int* __restrict__ slot_mapping) {
+    __shared__ float buf[4][QKN_MAXD];
+    const long t = blockIdx.x;
+    const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int pos = positions[t];
+    const int half = dims / 2;
+    const int slot = slot_mapping[t];
+    const long blk = slot / bs, off = slot % bs;
+    float* nb = buf[wid];
+    for (int hh = wid; hh < H + G; hh += 4) {
+        const bool is_q = hh < H;
+        const int g = hh - H;
+        const T* src = is_q ? q + t * q_tok + (long)hh * D
+                            : k + t * k_tok + (long)g * D;
+        const float* w = is_q ? wq : wk;
+        float ss = 0.f;
+        for (int i = lane; i < D; i += WAVE) {
+            const float x = ldf(src + i);
+            nb[i] = x;
+            ss += x * x;
+        }
+        const float r = 1.f / sqrtf(wave_sum(ss) / (float)D + eps);
+        const float mul = is_q ? q_mult[hh] : 1.f;
+        T* dst = is_q ? q + t * q_tok + (long)hh * D
+                      : k_cache + ((blk * G + g) * bs + off) * D;
+        T* vdst = is_q ? nullptr : v_cache + ((blk * G + g) * bs + off) * D;
+        // every lane has written its nb entries before any lane reads a
+        // partner's: the wave_sum above is a full-wave exchange, and the
+        // LDS writes of a wave complete in order before its later reads
+        WAVE_LDS_SYNC();
+        for (int i = lane; i < D; i += WAVE) {
+            const float x = nb[i];
+            float y = x * r * w[i];
+            if (i < dims) {
+                const int j = i < half ? i : i - half;
+                const int pi = i < half ? i + half : i - half;
+                const float yp = nb[pi] * r * w[pi];
+                const float c = cos_t[(long)pos * half + j];
+                const float s = sin_t[(long)pos * half + j];
+                y = i < half ? y * c - yp * s : y * c + yp * s;
+            }
+            stf(dst + i, y * mul);
+            if (vdst) stf(vdst + i, x);
+        }
+        WAVE_LDS_SYNC();
+    }
+}
 
 // ------------------------------------------------------------- launchers
 // dtype codes: 0 = bf16 (ushort bits), 1 = fp32
@@ -413,44 +618,161 @@ extern "C" void launch_clamped_glu(const void* gu, void* y, long rows, long I,
             (const unsigned short*)gu, (unsigned short*)y, rows, I, limit, alpha);
 }
 
+template <typename T, typename OT, bool RES, bool SILU>
+static void conv_dispatch(const void* h, long hs, const float* w, void* state,
+                          const int* state_slots, const int* cu,
+                          const int* seq_idx, const int* positions, void* out,
+                          long T_, int B, int C, int K, bool vec4,
+                          hipStream_t s) {
+    const int th = C >= 256 ? 256 : 64;
+    const int vec = vec4 ? 4 : 1;
+    const int lanes = (C + vec - 1) / vec;
+    const dim3 g1((unsigned)T_, (lanes + th - 1) / th), g2(B, (C + th - 1) / th);
+    if (vec4)
+        canon_conv_kernel<T, OT, 4, RES, SILU><<<g1, th, 0, s>>>(
+            (const T*)h, hs, w, (const T*)state, state_slots, cu, seq_idx,
+            positions, (OT*)out, C, K);
+    else
+        canon_conv_kernel<T, OT, 1, RES, SILU><<<g1, th, 0, s>>>(
+            (const T*)h, hs, w, (const T*)state, state_slots, cu, seq_idx,
+            positions, (OT*)out, C, K);
+    if (K > 0)
+        canon_state_kernel<T><<<g2, th, 0, s>>>(
+            (const T*)h, hs, (T*)state, state_slots, cu, C, K);
+}
+
+// h + conv(h), same dtype out (the sandwich layers' whole-width conv)
 extern "C" void launch_canon_conv(const void* h, const float* w, void* state,
                                   const int* state_slots, const int* cu,
                                   const int* seq_idx, const int* positions,
                                   void* out, long T, int B, int C, int K,
                                   int f32, hipStream_t s) {
     if (T == 0) return;
-    const int th = C >= 256 ? 256 : 64;
-    const int vec = C % 4 == 0 ? 4 : 1;
-    const int lanes = (C + vec - 1) / vec;
-    const dim3 g1((unsigned)T, (lanes + th - 1) / th), g2(B, (C + th - 1) / th);
-    if (f32) {
-        if (vec == 4)
-            canon_conv_kernel<float, 4><<<g1, th, 0, s>>>(
-                (const float*)h, w, (const float*)state, state_slots, cu,
-                seq_idx, positions, (float*)out, C, K);
-        else
-            canon_conv_kernel<float, 1><<<g1, th, 0, s>>>(
-                (const float*)h, w, (const float*)state, state_slots, cu, seq_idx,
-                positions, (float*)out, C, K);
-        if (K > 0)
-            canon_state_kernel<float><<<g2, th, 0, s>>>(
-                (const float*)h, (float*)state, state_slots, cu, C, K);
-    } else {
-        if (vec == 4)
-            canon_conv_kernel<unsigned short, 4><<<g1, th, 0, s>>>(
-                (const unsigned short*)h, w, (const unsigned short*)state,
-                state_slots, cu, seq_idx, positions, (unsigned short*)out, C,
-                K);
-        else
-            canon_conv_kernel<unsigned short, 1><<<g1, th, 0, s>>>(
-                (const unsigned short*)h, w, (const unsigned short*)state,
-                state_slots, cu, seq_idx, positions, (unsigned short*)out, C,
-                K);
-        if (K > 0)
-            canon_state_kernel<unsigned short><<<g2, th, 0, s>>>(
-                (const unsigned short*)h, (unsigned short*)state, state_slots,
-                cu, C, K);
-    }
+    const bool v4 = C % 4 == 0;
+    if (f32)
+        conv_dispatch<float, float, true, false>(
+            h, C, w, state, state_slots, cu, seq_idx, positions, out, T, B, C,
+            K, v4, s);
+    else
+        conv_dispatch<unsigned short, unsigned short, true, false>(
+            h, C, w, state, state_slots, cu, seq_idx, positions, out, T, B, C,
+            K, v4, s);
+}
+
+// conv(h) [silu] -> fp32, h a column slice with row stride hs
+extern "C" void launch_short_conv(const void* h, long hs, const float* w,
+                                  void* state, const int* state_slots,
+                                  const int* cu, const int* seq_idx,
+                                  const int* positions, float* out, long T,
+                                  int B, int C, int K, int silu, int vec4,
+                                  int f32, hipStream_t s) {
+    if (T == 0) return;
+#define SC_CALL(TT, SI)                                                       \
+    conv_dispatch<TT, float, false, SI>(h, hs, w, state, state_slots, cu,     \
+                                        seq_idx, positions, out, T, B, C, K,  \
+                                        vec4 != 0, s)
+    if (f32) { if (silu) SC_CALL(float, true); else SC_CALL(float, false); }
+    else if (silu) SC_CALL(unsigned short, true);
+    else SC_CALL(unsigned short, false);
+#undef SC_CALL
+}
+
+extern "C" void launch_add_rmsnorm_w(float* resid, const void* y,
+                                     const float* w, void* out, long T, int W,
+                                     float eps, int y_f32, int out_f32,
+                                     hipStream_t s) {
+    if (T == 0) return;
+    const size_t sh = (size_t)W * sizeof(float);
+#define ARW(YT, OT)                                                           \
+    do {                                                                      \
+        if (W % 4 == 0)                                                       \
+            add_rmsnorm_w_kernel<YT, OT, 4><<<T, row_threads(W / 4), sh, s>>>(\
+                resid, (const YT*)y, w, (OT*)out, W, eps);                    \
+        else                                                                  \
+            add_rmsnorm_w_kernel<YT, OT, 1><<<T, row_threads(W), sh, s>>>(    \
+                resid, (const YT*)y, w, (OT*)out, W, eps);                    \
+    } while (0)
+    if (y_f32 && out_f32) ARW(float, float);
+    else if (y_f32) ARW(float, unsigned short);
+    else if (out_f32) ARW(unsigned short, float);
+    else ARW(unsigned short, unsigned short);
+#undef ARW
+}
+
+extern "C" void launch_relu2(const void* x, long xs, void* out, long os,
+                             long rows, int n, int vec4, int f32,
+                             hipStream_t s) {
+    if (rows == 0 || n == 0) return;
+    const int th = 256;
+    long blocks = (rows * (long)(vec4 ? n / 4 : n) + th - 1) / th;
+    if (blocks > 65536) blocks = 65536;
+#define R2(TT, V)                                                             \
+    relu2_kernel<TT, V><<<(int)blocks, th, 0, s>>>((const TT*)x, xs,          \
+                                                   (TT*)out, os, rows, n)
+    if (f32) { if (vec4) R2(float, 4); else R2(float, 1); }
+    else if (vec4) R2(unsigned short, 4);
+    else R2(unsigned short, 1);
+#undef R2
+}
+
+extern "C" void launch_head_gated_norm(const float* o, const float* w,
+                                       const void* gate, long gs, void* out,
+                                       long os, long T, int H, int Dv,
+                                       float eps, int sigmoid,
+                                       float out_scale, int f32,
+                                       hipStream_t s) {
+    const long rows = T * H;
+    if (rows == 0) return;
+    const int wpb = 4;
+    const unsigned blocks = (unsigned)((rows + wpb - 1) / wpb);
+    if (f32)
+        head_gated_norm_kernel<float><<<blocks, wpb * WAVE, 0, s>>>(
+            o, w, (const float*)gate, gs, (float*)out, os, rows, H, Dv, eps,
+            sigmoid, out_scale);
+    else
+        head_gated_norm_kernel<unsigned short><<<blocks, wpb * WAVE, 0, s>>>(
+            o, w, (const unsigned short*)gate, gs, (unsigned short*)out, os,
+            rows, H, Dv, eps, sigmoid, out_scale);
+}
+
+extern "C" void launch_delta_gates(float* qk, long qs, int NQ, int D,
+                                   const void* b, long bs, const void* a,
+                                   long as, const float* dt_bias,
+                                   const float* rate, float* beta, float* g,
+                                   long T, int H, int per_head, int f32,
+                                   hipStream_t s) {
+    if (T == 0) return;
+    if (f32)
+        delta_gates_kernel<float><<<T, 256, 0, s>>>(
+            qk, qs, NQ, D, (const float*)b, bs, (const float*)a, as, dt_bias,
+            rate, beta, g, H, per_head);
+    else
+        delta_gates_kernel<unsigned short><<<T, 256, 0, s>>>(
+            qk, qs, NQ, D, (const unsigned short*)b, bs,
+            (const unsigned short*)a, as, dt_bias, rate, beta, g, H, per_head);
+}
+
+// returns nonzero when the head dim exceeds 512
+extern "C" int launch_qk_norm_rope_store(
+    void* q, long q_tok, int H, const void* k, long k_tok, int G, int D,
+    const float* wq, const float* wk, float eps, int dims,
+    const int* positions, const float* cos_t, const float* sin_t,
+    const float* q_mult, void* k_cache, void* v_cache, int bs,
+    const int* slot_mapping, long T, int f32, hipStream_t s) {
+    if (D > QKN_MAXD) return 1;
+    if (T == 0) return 0;
+    if (f32)
+        qk_norm_rope_store_kernel<float><<<T, 256, 0, s>>>(
+            (float*)q, q_tok, H, (const float*)k, k_tok, G, D, wq, wk, eps,
+            dims, positions, cos_t, sin_t, q_mult, (float*)k_cache,
+            (float*)v_cache, bs, slot_mapping);
+    else
+        qk_norm_rope_store_kernel<unsigned short><<<T, 256, 0, s>>>(
+            (unsigned short*)q, q_tok, H, (const unsigned short*)k, k_tok, G,
+            D, wq, wk, eps, dims, positions, cos_t, sin_t, q_mult,
+            (unsigned short*)k_cache, (unsigned short*)v_cache, bs,
+            slot_mapping);
+    return 0;
 }
 
 extern "C" void launch_latent_rope_store(

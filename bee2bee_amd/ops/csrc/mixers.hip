@@ -477,10 +477,30 @@ DEV_INLINE bool li_segment(const int* __restrict__ cu, int B, int seg,
     return false;
 }
 
-template <typename T, int DPT, int MODE>
+//
+// FORM 0 (lightning): q, k, v enter as silu of the projections.
+// FORM 1 (retention): q and k are rotated by position — coordinate i of the
+// first `rdims` pairs with i + rdims/2, angle from the fp32 cos/sin tables
+// [max_pos, rdims/2] — k is also multiplied by k_scale, v enters as is.
+template <typename T, int FORM>
+DEV_INLINE float li_load_qk(const T* __restrict__ row, int d, int rdims,
+                            const float* __restrict__ cs,
+                            const float* __restrict__ sn) {
+    const float x = ldf(row + d);
+    if (FORM == 0) return silu_f(x);
+    if (d >= rdims) return x;
+    const int half = rdims / 2;
+    const int j = d < half ? d : d - half;
+    const float y = ldf(row + (d < half ? d + half : d - half));
+    return d < half ? x * cs[j] - y * sn[j] : x * cs[j] + y * sn[j];
+}
+
+template <typename T, int DPT, int MODE, int FORM>
 __global__ void __launch_bounds__(LI_COLS * LI_GROUPS)
 lightning_kernel(const T* __restrict__ q, const T* __restrict__ k,
                  const T* __restrict__ v, long tok_stride,
+                 const float* __restrict__ cos_t,
+                 const float* __restrict__ sin_t, int rdims, float k_scale,
                  const float* __restrict__ decay,
                  float* __restrict__ state,        // [slots, H, D, Dv]
                  const int* __restrict__ state_slots,
@@ -526,17 +546,31 @@ lightning_kernel(const T* __restrict__ q, const T* __restrict__ k,
         const int n = min(LI_TB, hi - t0);
         for (int idx = threadIdx.x; idx < n * DMAX; idx += nth) {
             const int tt = idx / DMAX, d = idx - tt * DMAX;
-            const long base = (long)(t0 + tt) * tok_stride + (long)h * D + d;
-            qs[tt][d] = d < D ? silu_f(ldf(q + base)) : 0.f;
-            if (MODE != 2) ks[tt][d] = d < D ? silu_f(ldf(k + base)) : 0.f;
+            const long base = (long)(t0 + tt) * tok_stride + (long)h * D;
+            const float* cs = nullptr;
+            const float* sn = nullptr;
+            if (FORM == 1 && rdims > 0) {
+                const long pr = (long)positions[t0 + tt] * (rdims / 2);
+                cs = cos_t + pr;
+                sn = sin_t + pr;
+            }
+            qs[tt][d] = d < D ? li_load_qk<T, FORM>(q + base, d, rdims, cs, sn)
+                              : 0.f;
+            if (MODE != 2)
+                ks[tt][d] = d < D ? li_load_qk<T, FORM>(k + base, d, rdims, cs,
+                                                        sn) * k_scale
+                                  : 0.f;
         }
         if (MODE != 2) {
             for (int idx = threadIdx.x; idx < n * LI_COLS; idx += nth) {
                 const int tt = idx / LI_COLS, c = idx - tt * LI_COLS;
-                vs[tt][c] = (c0 + c < Dv)
-                    ? silu_f(ldf(v + (long)(t0 + tt) * tok_stride +
-                                 (long)h * Dv + c0 + c))
-                    : 0.f;
+                float vv = 0.f;
+                if (c0 + c < Dv) {
+                    vv = ldf(v + (long)(t0 + tt) * tok_stride + (long)h * Dv +
+                             c0 + c);
+                    if (FORM == 0) vv = silu_f(vv);
+                }
+                vs[tt][c] = vv;
             }
         }
         __syncthreads();
@@ -611,6 +645,299 @@ __global__ void lightning_scan_kernel(const float* __restrict__ decay,
         S = expf(log_lam * (float)n) * S + local;
     }
     *slot = S;
+}
+
+// ------------------------------------------------------------ delta rule
+// Gated delta rule on a memory M (key rows x value columns), fp32, per
+// token:  M <- g * M;  delta = beta (v - M^T k);  M <- M + k delta^T;
+// y = M^T q.  Since y = (gM)^T q + delta (k . q), both sums over the key
+// axis run on the faded memory in ONE pass.
+// A workgroup is ONE wave that owns DR_CW columns of one (sequence, value
+// head) state: lane (r, c) keeps rows [r*DPT, (r+1)*DPT) of column c in
+// registers, the DR_RG row groups are combined with two xor-shuffles, and
+// nothing but the staging of DR_TB tokens' q/k/g/v/beta through LDS needs a
+// barrier. Columns evolve independently -> sequences x heads x Dv/DR_CW
+// waves. Tokens are walked in order (the update of token t reads the state
+// token t-1 left).
+constexpr int DR_RG = 4;
+constexpr int DR_CW = WAVE / DR_RG;
+constexpr int DR_TB = 8;
+
+template <int DPT, bool CHDEC>
+__global__ void __launch_bounds__(WAVE)
+delta_rule_kernel(const float* __restrict__ q, const float* __restrict__ k,
+                  long qk_tok, const float* __restrict__ v, long v_tok,
+                  const float* __restrict__ beta,   // [Tn, H]
+                  const float* __restrict__ g,      // [Tn, H] | [Tn, H, D]
+                  float* __restrict__ state,        // [slots, H, D, Dv]
+                  const int* __restrict__ state_slots,
+                  const int* __restrict__ cu,
+                  const int* __restrict__ positions,
+                  float* __restrict__ out,          // [Tn, H, Dv]
+                  int H, int G, int D, int Dv) {
+    constexpr int DMAX = DPT * DR_RG;
+    __shared__ float qs[DR_TB][DMAX];
+    __shared__ float ks[DR_TB][DMAX];
+    __shared__ float gs[DR_TB][CHDEC ? DMAX : 1];
+    __shared__ float vs[DR_TB][DR_CW];
+    __shared__ float bs[DR_TB];
+    const int b = blockIdx.x, h = blockIdx.y;
+    const int lo = cu[b], hi = cu[b + 1];
+    if (hi <= lo) return;
+    const int lane = threadIdx.x;
+    const int r = lane / DR_CW, c = lane % DR_CW;
+    const int c0 = blockIdx.z * DR_CW;
+    const int dv = c0 + c;
+    const bool live = dv < Dv;
+    const int d0 = r * DPT;
+    const int kvh = h / (H / G);
+    float* st = state + (((long)state_slots[b] * H + h) * D) * Dv + dv;
+    const bool fresh = positions[lo] == 0;
+    float s[DPT];
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) {
+        const int d = d0 + i;
+        s[i] = (!fresh && live && d < D) ? st[(long)d * Dv] : 0.f;
+    }
+    for (int t0 = lo; t0 < hi; t0 += DR_TB) {
+        const int n = min(DR_TB, hi - t0);
+        for (int idx = lane; idx < n * DMAX; idx += WAVE) {
+            const int tt = idx / DMAX, d = idx - tt * DMAX;
+            const long base = (long)(t0 + tt) * qk_tok + (long)kvh * D + d;
+            qs[tt][d] = d < D ? q[base] : 0.f;
+            ks[tt][d] = d < D ? k[base] : 0.f;
+            if (CHDEC)
+                gs[tt][d] = d < D ? g[((long)(t0 + tt) * H + h) * D + d] : 1.f;
+        }
+        for (int idx = lane; idx < n * DR_CW; idx += WAVE) {
+            const int tt = idx / DR_CW, cc = idx - tt * DR_CW;
+            vs[tt][cc] = (c0 + cc < Dv)
+                ? v[(long)(t0 + tt) * v_tok + (long)h * Dv + c0 + cc] : 0.f;
+        }
+        if (lane < n) {
+            bs[lane] = beta[(long)(t0 + lane) * H + h];
+            if (!CHDEC) gs[lane][0] = g[(long)(t0 + lane) * H + h];
+        }
+        __syncthreads();
+        for (int tt = 0; tt < n; ++tt) {
+            float ka = 0.f, kb = 0.f, qa = 0.f, qb = 0.f, kq = 0.f;
+            const float gsc = CHDEC ? 1.f : gs[tt][0];
+#pragma unroll
+            for (int i = 0; i < DPT; i += 2) {
+                const float k0 = ks[tt][d0 + i], q0 = qs[tt][d0 + i];
+                const float s0 = s[i] * (CHDEC ? gs[tt][d0 + i] : gsc);
+                s[i] = s0;
+                ka += k0 * s0;
+                qa += q0 * s0;
+                kq += k0 * q0;
+                if (i + 1 < DPT) {
+                    const float k1 = ks[tt][d0 + i + 1];
+                    const float q1 = qs[tt][d0 + i + 1];
+                    const float s1 =
+                        s[i + 1] * (CHDEC ? gs[tt][d0 + i + 1] : gsc);
+                    s[i + 1] = s1;
+                    kb += k1 * s1;
+                    qb += q1 * s1;
+                    kq += k1 * q1;
+                }
+            }
+            float kS = ka + kb, qS = qa + qb;
+#pragma unroll
+            for (int off = DR_CW; off < WAVE; off <<= 1) {
+                kS += __shfl_xor(kS, off);
+                qS += __shfl_xor(qS, off);
+                kq += __shfl_xor(kq, off);
+            }
+            const float u = bs[tt] * (vs[tt][c] - kS);
+#pragma unroll
+            for (int i = 0; i < DPT; ++i) s[i] += ks[tt][d0 + i] * u;
+            if (r == 0 && live)
+                out[((long)(t0 + tt) * H + h) * Dv + dv] = qS + u * kq;
+        }
+        __syncthreads();
+    }
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < DPT; ++i) {
+            const int d = d0 + i;
+            if (d < D) st[(long)d * Dv] = s[i];
+        }
+    }
+}
+
+// ------------------------------------------------ attention with a sink
+// Causal grouped-query softmax attention over paged keys/values
+// [n_blocks, G, bs, D|Dv], any head size up to SA_MAXD, bf16 or fp32 pages.
+// One wave per (token, query head, key split): tiles of 64 keys — for the
+// scores a lane owns ONE key and walks its row against the query held in
+// LDS (fp32), the tile's max/sum are wave reductions, and for the weighted
+// value sum lanes own output coordinates while the weights are broadcast
+// lane by lane. Scores, weights and accumulators are fp32; every score
+// multiplier is already in q. The softmax denominator also counts
+// exp(sink[h]) once when sink is given. Row t at position p sees cached
+// positions j <= p (j > p - window when window > 0). With gridDim.z > 1
+// each split writes its (max, sum, partial) and sink_attn_combine merges.
+constexpr int SA_WAVES = 4;
+constexpr int SA_MAXD = 256;
+
+template <typename T>
+DEV_INLINE float sa_dot(const T* __restrict__ kr, const float* __restrict__ qv,
+                        int D);
+template <>
+DEV_INLINE float sa_dot<float>(const float* __restrict__ kr,
+                               const float* __restrict__ qv, int D) {
+    float a = 0.f, b = 0.f;
+    if (D % 4 == 0) {
+        for (int d = 0; d < D; d += 4) {
+            const f32x4 x = *reinterpret_cast<const f32x4*>(kr + d);
+            a += x[0] * qv[d] + x[2] * qv[d + 2];
+            b += x[1] * qv[d + 1] + x[3] * qv[d + 3];
+        }
+    } else {
+        for (int d = 0; d < D; ++d) a += kr[d] * qv[d];
+    }
+    return a + b;
+}
+template <>
+DEV_INLINE float sa_dot<unsigned short>(const unsigned short* __restrict__ kr,
+                                        const float* __restrict__ qv, int D) {
+    float a = 0.f, b = 0.f;
+    if (D % 8 == 0) {
+        for (int d = 0; d < D; d += 8) {
+            float x[8];
+            load_bf16x8(kr + d, x);
+#pragma unroll
+            for (int j = 0; j < 8; j += 2) {
+                a += x[j] * qv[d + j];
+                b += x[j + 1] * qv[d + j + 1];
+            }
+        }
+    } else {
+        for (int d = 0; d < D; ++d) a += bf2f(kr[d]) * qv[d];
+    }
+    return a + b;
+}
+
+template <typename T, int DPL>
+__global__ void __launch_bounds__(SA_WAVES * WAVE)
+sink_attn_kernel(const T* __restrict__ q, long q_tok,
+                 const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                 const int* __restrict__ block_table, int bt_stride,
+                 const int* __restrict__ positions,
+                 const int* __restrict__ seq_idx,
+                 const float* __restrict__ sink, T* __restrict__ out,
+                 long out_tok, float out_scale, float* __restrict__ part_acc,
+                 float* __restrict__ part_ml, int Tn, int H, int G, int D,
+                 int Dv, int bs, int window) {
+    __shared__ float qs[SA_WAVES][SA_MAXD];
+    const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int t = blockIdx.x, h = blockIdx.y * SA_WAVES + wid;
+    if (h >= H) return;      // no workgroup barrier below
+    const int split = blockIdx.z, nsplit = gridDim.z;
+    const int p = positions[t];
+    const int g = h / (H / G);
+    const int lo = window > 0 ? max(0, p - window + 1) : 0;
+    const int per = (p + 1 - lo + nsplit - 1) / nsplit;
+    const int klo = lo + split * per, khi = min(p + 1, klo + per);
+    float* qv = qs[wid];
+    for (int i = lane; i < D; i += WAVE)
+        qv[i] = ldf(q + (long)t * q_tok + (long)h * D + i);
+    WAVE_LDS_SYNC();
+    const int* bt = block_table + (long)seq_idx[t] * bt_stride;
+    float m = -INFINITY, l = 0.f;
+    float acc[DPL];
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) acc[i] = 0.f;
+    for (int j0 = klo; j0 < khi; j0 += WAVE) {
+        const int j = j0 + lane;
+        const bool valid = j < khi;
+        int row = 0;
+        float sc = -INFINITY;
+        if (valid) {
+            row = (bt[j / bs] * G + g) * bs + j % bs;
+            sc = sa_dot<T>(k_cache + (long)row * D, qv, D);
+        }
+        const float m_new = fmaxf(m, wave_max(sc));
+        const float pj = valid ? expf(sc - m_new) : 0.f;
+        const float corr = expf(m - m_new);
+        l = l * corr + wave_sum(pj);
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) acc[i] *= corr;
+        const int nk = min(WAVE, khi - j0);
+        for (int jj = 0; jj < nk; ++jj) {
+            const float pb = __shfl(pj, jj);
+            const T* vr = v_cache + (long)__shfl(row, jj) * Dv;
+#pragma unroll
+            for (int i = 0; i < DPL; ++i) {
+                const int d = lane + i * WAVE;
+                if (d < Dv) acc[i] += pb * ldf(vr + d);
+            }
+        }
+        m = m_new;
+    }
+    if (nsplit == 1) {
+        float L = l, w = 1.f;
+        if (sink) {
+            const float sk = sink[h];
+            const float M = fmaxf(m, sk);
+            w = expf(m - M);
+            L = l * w + expf(sk - M);
+        }
+        const float rcp = L > 0.f ? out_scale * w / L : 0.f;
+        T* o = out + (long)t * out_tok + (long)h * Dv;
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) {
+            const int d = lane + i * WAVE;
+            if (d < Dv) stf(o + d, acc[i] * rcp);
+        }
+        return;
+    }
+    const long prow = ((long)split * H + h) * Tn + t;
+    if (lane == 0) {
+        part_ml[prow * 2] = m;
+        part_ml[prow * 2 + 1] = l;
+    }
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) {
+        const int d = lane + i * WAVE;
+        if (d < Dv) part_acc[prow * Dv + d] = acc[i];
+    }
+}
+
+// merge of the key splits: wave per (token, head)
+template <typename T>
+__global__ void __launch_bounds__(SA_WAVES * WAVE)
+sink_attn_combine_kernel(const float* __restrict__ part_acc,
+                         const float* __restrict__ part_ml,
+                         const float* __restrict__ sink, T* __restrict__ out,
+                         long out_tok, float out_scale, int splits, int Tn,
+                         int H, int Dv) {
+    const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int t = blockIdx.x, h = blockIdx.y * SA_WAVES + wid;
+    if (h >= H) return;
+    float m = -INFINITY, l = 0.f;
+    if (lane < splits) {
+        const long row = ((long)lane * H + h) * Tn + t;
+        m = part_ml[row * 2];
+        l = part_ml[row * 2 + 1];
+    }
+    float M = wave_max(l > 0.f ? m : -INFINITY);
+    if (sink) M = fmaxf(M, sink[h]);
+    const float w = l > 0.f ? expf(m - M) : 0.f;
+    float L = wave_sum(l * w);
+    if (sink) L += expf(sink[h] - M);
+    const float rcp = L > 0.f ? out_scale / L : 0.f;
+    T* o = out + (long)t * out_tok + (long)h * Dv;
+    for (int d0 = 0; d0 < Dv; d0 += WAVE) {
+        const int d = d0 + lane;
+        float a = 0.f;
+        for (int z = 0; z < splits; ++z) {
+            const float wz = __shfl(w, z);
+            if (d < Dv)
+                a += part_acc[(((long)z * H + h) * Tn + t) * Dv + d] * wz;
+        }
+        if (d < Dv) stf(o + d, a * rcp);
+    }
 }
 
 }  // namespace
@@ -725,9 +1052,11 @@ extern "C" int launch_latent_attn_mfma(
 }
 
 #define LI_LAUNCH(N, MODE, GRID)                                              \
-    lightning_kernel<TT, N, MODE><<<GRID, LI_COLS * LI_GROUPS, 0, s>>>(       \
-        (const TT*)q, (const TT*)k, (const TT*)v, tok_stride, decay, state,   \
-        state_slots, cu, positions, out, ws, B, H, D, Dv)
+    lightning_kernel<TT, N, MODE, FORM>                                       \
+        <<<GRID, LI_COLS * LI_GROUPS, 0, s>>>(                                \
+            (const TT*)q, (const TT*)k, (const TT*)v, tok_stride, cos_t,      \
+            sin_t, rdims, k_scale, decay, state, state_slots, cu, positions,  \
+            out, ws, B, H, D, Dv)
 
 #define LI_CASE(N)                                                            \
     case N:                                                                   \
@@ -744,9 +1073,11 @@ extern "C" int launch_latent_attn_mfma(
 // n_seg = 0: one workgroup walks each whole chunk. n_seg > 0 (an upper bound
 // of the number of LI_SEG-token segments in the batch, ws sized for it):
 // segments run in parallel, a scan carries the state across them.
-template <typename TT>
+template <typename TT, int FORM>
 static int lightning_dispatch(const void* q, const void* k, const void* v,
-                              long tok_stride, const float* decay,
+                              long tok_stride, const float* cos_t,
+                              const float* sin_t, int rdims, float k_scale,
+                              const float* decay,
                               float* state, const int* state_slots,
                               const int* cu, const int* positions, float* out,
                               float* ws, int n_seg, int B, int H, int D,
@@ -767,20 +1098,113 @@ static int lightning_dispatch(const void* q, const void* k, const void* v,
 // returns nonzero when the key dim exceeds 256
 extern "C" int lightning_segment_tokens() { return LI_SEG; }
 
+// form 0: silu(q, k, v) (lightning); form 1: rotated q, k, scaled k, plain
+// v (retention; cos_t/sin_t may be null when rdims is 0)
 extern "C" int launch_lightning(const void* q, const void* k, const void* v,
                                 long tok_stride, const float* decay,
                                 float* state, const int* state_slots,
                                 const int* cu, const int* positions,
                                 float* out, float* ws, int n_seg, int B,
-                                int H, int D, int Dv, int f32,
-                                hipStream_t s) {
+                                int H, int D, int Dv, int f32, int form,
+                                const float* cos_t, const float* sin_t,
+                                int rdims, float k_scale, hipStream_t s) {
     if (B == 0) return 0;
+#define LI_DISPATCH(TT, FORM)                                                 \
+    lightning_dispatch<TT, FORM>(q, k, v, tok_stride, cos_t, sin_t, rdims,    \
+                                 k_scale, decay, state, state_slots, cu,      \
+                                 positions, out, ws, n_seg, B, H, D, Dv, s)
+    if (form == 0)
+        return f32 ? LI_DISPATCH(float, 0) : LI_DISPATCH(unsigned short, 0);
+    return f32 ? LI_DISPATCH(float, 1) : LI_DISPATCH(unsigned short, 1);
+#undef LI_DISPATCH
+}
+
+#define DR_CASE(N)                                                            \
+    case N:                                                                   \
+        if (chdec)                                                            \
+            delta_rule_kernel<N, true><<<grid, WAVE, 0, s>>>(                 \
+                q, k, qk_tok, v, v_tok, beta, g, state, state_slots, cu,      \
+                positions, out, H, G, D, Dv);                                 \
+        else                                                                  \
+            delta_rule_kernel<N, false><<<grid, WAVE, 0, s>>>(                \
+                q, k, qk_tok, v, v_tok, beta, g, state, state_slots, cu,      \
+                positions, out, H, G, D, Dv);                                 \
+        break;
+
+// returns nonzero when the key dim exceeds 256
+extern "C" int launch_delta_rule(const float* q, const float* k, long qk_tok,
+                                 const float* v, long v_tok,
+                                 const float* beta, const float* g, int chdec,
+                                 float* state, const int* state_slots,
+                                 const int* cu, const int* positions,
+                                 float* out, int B, int H, int G, int D,
+                                 int Dv, hipStream_t s) {
+    if (B == 0) return 0;
+    const int need = (D + DR_RG - 1) / DR_RG;
+    const int sizes[] = {2, 4, 8, 16, 32, 64};
+    int dpt = 0;
+    for (int z : sizes)
+        if (z >= need) { dpt = z; break; }
+    if (!dpt) return 1;
+    const dim3 grid(B, H, (Dv + DR_CW - 1) / DR_CW);
+    switch (dpt) {
+        DR_CASE(2) DR_CASE(4) DR_CASE(8) DR_CASE(16) DR_CASE(32) DR_CASE(64)
+    }
+    return 0;
+}
+
+#define SA_CASE(N)                                                            \
+    case N:                                                                   \
+        sink_attn_kernel<TT, N><<<grid, SA_WAVES * WAVE, 0, s>>>(             \
+            (const TT*)q, q_tok, (const TT*)k_cache, (const TT*)v_cache,      \
+            block_table, bt_stride, positions, seq_idx, sink, (TT*)out,       \
+            out_tok, out_scale, part_acc, part_ml, Tn, H, G, D, Dv, bs,       \
+            window);                                                          \
+        break;
+
+template <typename TT>
+static int sink_attn_dispatch(const void* q, long q_tok, const void* k_cache,
+                              const void* v_cache, const int* block_table,
+                              int bt_stride, const int* positions,
+                              const int* seq_idx, const float* sink,
+                              void* out, long out_tok, float out_scale,
+                              float* part_acc, float* part_ml, int splits,
+                              int Tn, int H, int G, int D, int Dv, int bs,
+                              int window, hipStream_t s) {
+    const int dpl = (Dv + WAVE - 1) / WAVE;
+    const dim3 grid(Tn, (H + SA_WAVES - 1) / SA_WAVES, splits);
+    switch (dpl) {
+        SA_CASE(1) SA_CASE(2) SA_CASE(3) SA_CASE(4)
+        default: return 1;
+    }
+    if (splits > 1) {
+        const dim3 g2(Tn, (H + SA_WAVES - 1) / SA_WAVES);
+        sink_attn_combine_kernel<TT><<<g2, SA_WAVES * WAVE, 0, s>>>(
+            part_acc, part_ml, sink, (TT*)out, out_tok, out_scale, splits, Tn,
+            H, Dv);
+    }
+    return 0;
+}
+
+// returns nonzero when a head size exceeds 256
+extern "C" int launch_sink_attn(const void* q, long q_tok,
+                                const void* k_cache, const void* v_cache,
+                                const int* block_table, int bt_stride,
+                                const int* positions, const int* seq_idx,
+                                const float* sink, void* out, long out_tok,
+                                float out_scale, float* part_acc,
+                                float* part_ml, int splits, int Tn, int H,
+                                int G, int D, int Dv, int bs, int window,
+                                int f32, hipStream_t s) {
+    if (D > SA_MAXD || Dv > SA_MAXD) return 1;
+    if (Tn == 0) return 0;
     if (f32)
-        return lightning_dispatch<float>(q, k, v, tok_stride, decay, state,
-                                         state_slots, cu, positions, out, ws,
-                                         n_seg, B, H, D, Dv, s);
-    return lightning_dispatch<unsigned short>(q, k, v, tok_stride, decay,
-                                              state, state_slots, cu,
-                                              positions, out, ws, n_seg, B, H,
-                                              D, Dv, s);
+        return sink_attn_dispatch<float>(
+            q, q_tok, k_cache, v_cache, block_table, bt_stride, positions,
+            seq_idx, sink, out, out_tok, out_scale, part_acc, part_ml, splits,
+            Tn, H, G, D, Dv, bs, window, s);
+    return sink_attn_dispatch<unsigned short>(
+        q, q_tok, k_cache, v_cache, block_table, bt_stride, positions,
+        seq_idx, sink, out, out_tok, out_scale, part_acc, part_ml, splits, Tn,
+        H, G, D, Dv, bs, window, s);
 }
