@@ -133,7 +133,13 @@ __global__ __launch_bounds__(64) void attn_prefill_basic(
 #define PF_TN 64                     // kv tile (4 x 16-key fragments)
 #define PF_PAD 8                     // LDS row padding (bf16 elems)
 
-template <int HD, bool PAGED, typename KVT>
+// HILO: the softmax weights enter the P V product as a bf16 PAIR (hi + lo,
+// two MFMAs, ~16 mantissa bits) instead of one bf16 rounding — for designs
+// whose attention weights are 32-bit quantities. sink (optional, [nq] fp32):
+// a per-head logit counted once in the softmax denominator, with no key and
+// no value. The output row of token t, head h starts at out + t*s_o + h*HD
+// and is multiplied by out_scale.
+template <int HD, bool PAGED, typename KVT, bool HILO = false>
 __global__ __launch_bounds__(256) void attn_prefill_mfma(
     const unsigned short* __restrict__ q,
     const KVT* __restrict__ k,  // PAGED: k_cache [nb,nkv,bs,hd]
@@ -143,7 +149,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
     const int* __restrict__ seq_lens,      // PAGED only
     unsigned short* __restrict__ out,
     int nq, int nkv, long s_q, long s_k, long s_v, int W, int bs,
-    float scale) {
+    float scale, const float* __restrict__ sink, float out_scale, long s_o) {
     constexpr int KSTEPS = HD / 32;
     const int seq = blockIdx.z;
     const int h = blockIdx.y;
@@ -169,7 +175,8 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
     // larger one and a K-sized carve would let P overwrite V^T.
     constexpr int VT_STRIDE = PF_TN + PF_PAD;
     constexpr int K_ELEMS = PF_TN * (HD + PF_PAD);
-    constexpr int P_ELEMS = PF_TM * VT_STRIDE;
+    constexpr int P_TILE = PF_TM * VT_STRIDE;
+    constexpr int P_ELEMS = P_TILE * (HILO ? 2 : 1);
     constexpr int VT_OFF = (K_ELEMS > P_ELEMS ? K_ELEMS : P_ELEMS);
     unsigned short* k_s = reinterpret_cast<unsigned short*>(smem_raw);
     unsigned short* vt_s = k_s + VT_OFF;
@@ -298,8 +305,11 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
                 float pv = __expf(sfrag[f][r] - m_run[r]);
                 if (sfrag[f][r] <= -1e29f) pv = 0.f;
                 psum[r] += pv;
-                p_s[(wid * PF_QROWS + lg * 4 + r) * VT_STRIDE + f * 16 + li] =
-                    f2bf(pv);
+                const int pi =
+                    (wid * PF_QROWS + lg * 4 + r) * VT_STRIDE + f * 16 + li;
+                const unsigned short hi = f2bf(pv);
+                p_s[pi] = hi;
+                if (HILO) p_s[P_TILE + pi] = f2bf(pv - bf2f(hi));
             }
         }
         // row sum across group lanes
@@ -322,10 +332,14 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
         // share the LDS buffer -> sync so K-tile reuse is safe)
         __syncthreads();
         bf16x8 a_p[PF_TN / 32];  // A k-dim = keys: 32 keys per fragment
+        bf16x8 a_pl[HILO ? PF_TN / 32 : 1];
 #pragma unroll
-        for (int ks2 = 0; ks2 < PF_TN / 32; ++ks2)
-            a_p[ks2] = *reinterpret_cast<const bf16x8*>(
-                p_s + (wid * PF_QROWS + li) * VT_STRIDE + ks2 * 32 + lg * 8);
+        for (int ks2 = 0; ks2 < PF_TN / 32; ++ks2) {
+            const int pi = (wid * PF_QROWS + li) * VT_STRIDE + ks2 * 32 + lg * 8;
+            a_p[ks2] = *reinterpret_cast<const bf16x8*>(p_s + pi);
+            if (HILO)
+                a_pl[ks2] = *reinterpret_cast<const bf16x8*>(p_s + P_TILE + pi);
+        }
 #pragma unroll
         for (int nb = 0; nb < HD / 16; ++nb) {
 #pragma unroll
@@ -334,6 +348,9 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
                     vt_s + (nb * 16 + li) * VT_STRIDE + ks2 * 32 + lg * 8);
                 o_acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                     a_p[ks2], bv, o_acc[nb], 0, 0, 0);
+                if (HILO)
+                    o_acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        a_pl[ks2], bv, o_acc[nb], 0, 0, 0);
             }
         }
     }
@@ -344,18 +361,26 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma(
     for (int r = 0; r < 4; ++r) {
         const int qrow = orow_base + lg * 4 + r;
         if (qrow >= QL) continue;
-        const float inv = (l_run[r] > 0.f) ? 1.f / l_run[r] : 0.f;
-        unsigned short* orow = out + ((long)(s0 + qrow) * nq + h) * HD;
+        float lsum = l_run[r], w = out_scale;
+        if (sink) {
+            const float sk = sink[h];
+            const float M = fmaxf(m_run[r], sk);
+            const float e = __expf(m_run[r] - M);
+            lsum = lsum * e + __expf(sk - M);
+            w *= e;
+        }
+        const float inv = (lsum > 0.f) ? w / lsum : 0.f;
+        unsigned short* orow = out + (long)(s0 + qrow) * s_o + (long)h * HD;
 #pragma unroll
         for (int nb = 0; nb < HD / 16; ++nb)
             orow[nb * 16 + li] = f2bf(o_acc[nb][r] * inv);
     }
 }
 
-static int prefill_mfma_smem(int hd) {
-    // LDS: max(K tile, P tile) + V^T tile, bf16; must match VT_OFF
+static int prefill_mfma_smem(int hd, int hilo = 0) {
+    // LDS: max(K tile, P tile(s)) + V^T tile, bf16; must match VT_OFF
     const int k_bytes = PF_TN * (hd + PF_PAD) * 2;
-    const int p_bytes = PF_TM * (PF_TN + PF_PAD) * 2;
+    const int p_bytes = PF_TM * (PF_TN + PF_PAD) * 2 * (hilo ? 2 : 1);
     const int vt_bytes = hd * (PF_TN + PF_PAD) * 2;
     return (k_bytes > p_bytes ? k_bytes : p_bytes) + vt_bytes;
 }
@@ -373,12 +398,12 @@ extern "C" void launch_attn_prefill(
             hipLaunchKernelGGL((attn_prefill_mfma<128, false, unsigned short>),
                                grid, dim3(256), smem, stream, q, k, v, cu,
                                nullptr, nullptr, out, nq, nkv, s_q, s_k, s_v,
-                               0, 0, scale);
+                               0, 0, scale, nullptr, 1.f, (long)nq * hd);
         else
             hipLaunchKernelGGL((attn_prefill_mfma<64, false, unsigned short>),
                                grid, dim3(256), smem, stream, q, k, v, cu,
                                nullptr, nullptr, out, nq, nkv, s_q, s_k, s_v,
-                               0, 0, scale);
+                               0, 0, scale, nullptr, 1.f, (long)nq * hd);
         return;
     }
     dim3 grid(nq, nseq);
@@ -409,12 +434,14 @@ extern "C" void launch_attn_prefill_paged(
                 hipLaunchKernelGGL((attn_prefill_mfma<128, true, KVT>), grid,  \
                                    dim3(256), smem, stream, q, kc, vc, cu,     \
                                    block_table, seq_lens, out, nq, nkv, s_q,   \
-                                   0, 0, W, bs, scale);                        \
+                                   0, 0, W, bs, scale, nullptr, 1.f,           \
+                                   (long)nq * hd);                             \
             else                                                               \
                 hipLaunchKernelGGL((attn_prefill_mfma<64, true, KVT>), grid,   \
                                    dim3(256), smem, stream, q, kc, vc, cu,     \
                                    block_table, seq_lens, out, nq, nkv, s_q,   \
-                                   0, 0, W, bs, scale);                        \
+                                   0, 0, W, bs, scale, nullptr, 1.f,           \
+                                   (long)nq * hd);                             \
             return;                                                            \
         }                                                                      \
         dim3 grid(nq, nseq);                                                   \
@@ -426,4 +453,35 @@ extern "C" void launch_attn_prefill_paged(
     if (fp8) PFP_LAUNCH(unsigned char);
     else PFP_LAUNCH(unsigned short);
 #undef PFP_LAUNCH
+}
+
+// Packed query chunks against the paged history with fp32-grade softmax
+// weights (bf16 hi+lo pair), an optional per-head sink logit, an output
+// scale and a strided output (a column slice of a wider buffer). bf16,
+// head size 64 or 128 (returns nonzero otherwise); scale is applied by the
+// caller (folded into q).
+extern "C" int launch_attn_prefill_paged_sink(
+    const unsigned short* q, long s_q, const unsigned short* k_cache,
+    const unsigned short* v_cache, const int* cu, const int* block_table,
+    const int* seq_lens, unsigned short* out, long s_o, int nseq, int nq,
+    int nkv, int hd, int W, int bs, int max_qlen, const float* sink,
+    float out_scale, hipStream_t stream) {
+    if (hd != 64 && hd != 128) return 1;
+    if (nseq == 0 || max_qlen == 0) return 0;
+    const int tiles = (max_qlen + PF_TM - 1) / PF_TM;
+    dim3 grid(tiles, nq, nseq);
+    const int smem = prefill_mfma_smem(hd, 1);
+    if (hd == 128)
+        hipLaunchKernelGGL(
+            (attn_prefill_mfma<128, true, unsigned short, true>), grid,
+            dim3(256), smem, stream, q, k_cache, v_cache, cu, block_table,
+            seq_lens, out, nq, nkv, s_q, 0, 0, W, bs, 1.f, sink, out_scale,
+            s_o);
+    else
+        hipLaunchKernelGGL(
+            (attn_prefill_mfma<64, true, unsigned short, true>), grid,
+            dim3(256), smem, stream, q, k_cache, v_cache, cu, block_table,
+            seq_lens, out, nq, nkv, s_q, 0, 0, W, bs, 1.f, sink, out_scale,
+            s_o);
+    return 0;
 }

@@ -66,6 +66,12 @@ int launch_delta_rule(const float*, const float*, long, const float*, long,
                       const float*, const float*, int, float*, const int*,
                       const int*, const int*, float*, int, int, int, int, int,
                       hipStream_t);
+int launch_attn_prefill_paged_sink(const unsigned short*, long,
+                                   const unsigned short*,
+                                   const unsigned short*, const int*,
+                                   const int*, const int*, unsigned short*,
+                                   long, int, int, int, int, int, int, int,
+                                   const float*, float, hipStream_t);
 int launch_sink_attn(const void*, long, const void*, const void*, const int*,
                      int, const int*, const int*, const float*, void*, long,
                      float, float*, float*, int, int, int, int, int, int, int,
@@ -661,10 +667,36 @@ void sink_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache,
         TORCH_CHECK(sink->numel() == H);
         sk = sink->data_ptr<float>();
     }
+    check_i32(cu, "cu_seqlens");
+    // bf16 prompt portions with head size 64/128 run on the matrix cores
+    // (the dense models' paged prefill kernel, with the weights as a bf16
+    // pair and the sink in its epilogue); single rows in the same step ride
+    // along. fp32, other head sizes, windows and pure decode steps take the
+    // generic kernel below.
+    if (c == 0 && max_qlen >= 16 && window == 0 && D == Dv &&
+        (D == 64 || D == 128)) {
+        const long B = cu.numel() - 1;
+        TORCH_CHECK(block_table.size(0) == B);
+        Tensor last = cu.slice(0, 1, B + 1).to(torch::kLong) - 1;
+        Tensor seq_lens =
+            (positions.index_select(0, last.clamp_min(0)) + 1)
+                .to(torch::kInt32);
+        const int rc = launch_attn_prefill_paged_sink(
+            (const unsigned short*)q.data_ptr(), q.stride(0),
+            (const unsigned short*)k_cache.data_ptr(),
+            (const unsigned short*)v_cache.data_ptr(), cu.data_ptr<int>(),
+            block_table.data_ptr<int>(), seq_lens.data_ptr<int>(),
+            (unsigned short*)out.data_ptr(), out.stride(0), (int)B, H, G, D,
+            (int)block_table.size(1), bs, (int)max_qlen, sk,
+            (float)out_scale, stream());
+        TORCH_CHECK(rc == 0, "sink_attn: matrix-core path refused a shape "
+                             "its guard admitted");
+        return;
+    }
     // few rows (decode): split each row's keys over more workgroups, at
     // least 128 keys per share of the longest context the tables can hold
     const long ctx = window > 0 ? window : block_table.size(1) * (long)bs;
-    long splits = 4096 / std::max<long>(1, (long)Tn * H);
+    long splits = 8192 / std::max<long>(1, (long)Tn * H);
     splits = std::min<long>({splits, 16, (ctx + 127) / 128});
     splits = std::max<long>(splits, 1);
     Tensor part_acc, part_ml;

@@ -676,9 +676,9 @@ delta_rule_kernel(const float* __restrict__ q, const float* __restrict__ k,
                   float* __restrict__ out,          // [Tn, H, Dv]
                   int H, int G, int D, int Dv) {
     constexpr int DMAX = DPT * DR_RG;
-    __shared__ float qs[DR_TB][DMAX];
-    __shared__ float ks[DR_TB][DMAX];
-    __shared__ float gs[DR_TB][CHDEC ? DMAX : 1];
+    __shared__ __attribute__((aligned(16))) float qs[DR_TB][DMAX];
+    __shared__ __attribute__((aligned(16))) float ks[DR_TB][DMAX];
+    __shared__ __attribute__((aligned(16))) float gs[DR_TB][CHDEC ? DMAX : 4];
     __shared__ float vs[DR_TB][DR_CW];
     __shared__ float bs[DR_TB];
     const int b = blockIdx.x, h = blockIdx.y;
@@ -720,26 +720,49 @@ delta_rule_kernel(const float* __restrict__ q, const float* __restrict__ k,
         }
         __syncthreads();
         for (int tt = 0; tt < n; ++tt) {
+            // this lane's slice of k, q (and the per-channel decay) into
+            // registers with 16-byte LDS reads; k is used twice
+            float kr[DPT], qr[DPT], gr[CHDEC ? DPT : 1];
+            if constexpr (DPT % 4 == 0) {
+#pragma unroll
+                for (int i = 0; i < DPT; i += 4) {
+                    const f32x4 a =
+                        *reinterpret_cast<const f32x4*>(&ks[tt][d0 + i]);
+                    const f32x4 b =
+                        *reinterpret_cast<const f32x4*>(&qs[tt][d0 + i]);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        kr[i + j] = a[j];
+                        qr[i + j] = b[j];
+                    }
+                    if constexpr (CHDEC) {
+                        const f32x4 e =
+                            *reinterpret_cast<const f32x4*>(&gs[tt][d0 + i]);
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) gr[i + j] = e[j];
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < DPT; ++i) {
+                    kr[i] = ks[tt][d0 + i];
+                    qr[i] = qs[tt][d0 + i];
+                    if constexpr (CHDEC) gr[i] = gs[tt][d0 + i];
+                }
+            }
+            if constexpr (!CHDEC) gr[0] = gs[tt][0];
             float ka = 0.f, kb = 0.f, qa = 0.f, qb = 0.f, kq = 0.f;
-            const float gsc = CHDEC ? 1.f : gs[tt][0];
 #pragma unroll
             for (int i = 0; i < DPT; i += 2) {
-                const float k0 = ks[tt][d0 + i], q0 = qs[tt][d0 + i];
-                const float s0 = s[i] * (CHDEC ? gs[tt][d0 + i] : gsc);
+                const float s0 = s[i] * gr[CHDEC ? i : 0];
+                const float s1 = s[i + 1] * gr[CHDEC ? i + 1 : 0];
                 s[i] = s0;
-                ka += k0 * s0;
-                qa += q0 * s0;
-                kq += k0 * q0;
-                if (i + 1 < DPT) {
-                    const float k1 = ks[tt][d0 + i + 1];
-                    const float q1 = qs[tt][d0 + i + 1];
-                    const float s1 =
-                        s[i + 1] * (CHDEC ? gs[tt][d0 + i + 1] : gsc);
-                    s[i + 1] = s1;
-                    kb += k1 * s1;
-                    qb += q1 * s1;
-                    kq += k1 * q1;
-                }
+                s[i + 1] = s1;
+                ka += kr[i] * s0;
+                kb += kr[i + 1] * s1;
+                qa += qr[i] * s0;
+                qb += qr[i + 1] * s1;
+                kq += kr[i] * qr[i] + kr[i + 1] * qr[i + 1];
             }
             float kS = ka + kb, qS = qa + qb;
 #pragma unroll
@@ -750,7 +773,7 @@ delta_rule_kernel(const float* __restrict__ q, const float* __restrict__ k,
             }
             const float u = bs[tt] * (vs[tt][c] - kS);
 #pragma unroll
-            for (int i = 0; i < DPT; ++i) s[i] += ks[tt][d0 + i] * u;
+            for (int i = 0; i < DPT; ++i) s[i] += kr[i] * u;
             if (r == 0 && live)
                 out[((long)(t0 + tt) * H + h) * Dv + dv] = qS + u * kq;
         }
@@ -780,45 +803,77 @@ delta_rule_kernel(const float* __restrict__ q, const float* __restrict__ k,
 constexpr int SA_WAVES = 4;
 constexpr int SA_MAXD = 256;
 
-template <typename T>
-DEV_INLINE float sa_dot(const T* __restrict__ kr, const float* __restrict__ qv,
-                        int D);
-template <>
-DEV_INLINE float sa_dot<float>(const float* __restrict__ kr,
-                               const float* __restrict__ qv, int D) {
-    float a = 0.f, b = 0.f;
+// scores of one key row against REP query vectors held in LDS (fp32)
+template <typename T, int REP>
+DEV_INLINE void sa_dots(const T* __restrict__ kr, const float* __restrict__ qv,
+                        int D, float* __restrict__ sc);
+template <int REP>
+DEV_INLINE void sa_dots_f32(const float* __restrict__ kr,
+                            const float* __restrict__ qv, int D,
+                            float* __restrict__ sc) {
     if (D % 4 == 0) {
         for (int d = 0; d < D; d += 4) {
             const f32x4 x = *reinterpret_cast<const f32x4*>(kr + d);
-            a += x[0] * qv[d] + x[2] * qv[d + 2];
-            b += x[1] * qv[d + 1] + x[3] * qv[d + 3];
+#pragma unroll
+            for (int r = 0; r < REP; ++r) {
+                const float* qr = qv + r * D + d;
+                sc[r] += x[0] * qr[0] + x[1] * qr[1] + x[2] * qr[2] +
+                         x[3] * qr[3];
+            }
         }
     } else {
-        for (int d = 0; d < D; ++d) a += kr[d] * qv[d];
+        for (int d = 0; d < D; ++d) {
+            const float x = kr[d];
+#pragma unroll
+            for (int r = 0; r < REP; ++r) sc[r] += x * qv[r * D + d];
+        }
     }
-    return a + b;
 }
-template <>
-DEV_INLINE float sa_dot<unsigned short>(const unsigned short* __restrict__ kr,
-                                        const float* __restrict__ qv, int D) {
-    float a = 0.f, b = 0.f;
+template <int REP>
+DEV_INLINE void sa_dots_bf16(const unsigned short* __restrict__ kr,
+                             const float* __restrict__ qv, int D,
+                             float* __restrict__ sc) {
     if (D % 8 == 0) {
         for (int d = 0; d < D; d += 8) {
             float x[8];
             load_bf16x8(kr + d, x);
 #pragma unroll
-            for (int j = 0; j < 8; j += 2) {
-                a += x[j] * qv[d + j];
-                b += x[j + 1] * qv[d + j + 1];
+            for (int r = 0; r < REP; ++r) {
+                const float* qr = qv + r * D + d;
+                float a = 0.f, b = 0.f;
+#pragma unroll
+                for (int j = 0; j < 8; j += 2) {
+                    a += x[j] * qr[j];
+                    b += x[j + 1] * qr[j + 1];
+                }
+                sc[r] += a + b;
             }
         }
     } else {
-        for (int d = 0; d < D; ++d) a += bf2f(kr[d]) * qv[d];
+        for (int d = 0; d < D; ++d) {
+            const float x = bf2f(kr[d]);
+#pragma unroll
+            for (int r = 0; r < REP; ++r) sc[r] += x * qv[r * D + d];
+        }
     }
-    return a + b;
 }
+template <typename T, int REP> struct SaDots;
+template <int REP> struct SaDots<float, REP> {
+    static DEV_INLINE void run(const float* kr, const float* qv, int D,
+                               float* sc) { sa_dots_f32<REP>(kr, qv, D, sc); }
+};
+template <int REP> struct SaDots<unsigned short, REP> {
+    static DEV_INLINE void run(const unsigned short* kr, const float* qv,
+                               int D, float* sc) {
+        sa_dots_bf16<REP>(kr, qv, D, sc);
+    }
+};
 
-template <typename T, int DPL>
+// A wave serves REP query heads that share one key/value head (REP divides
+// the group size), so each cached row is read once for all of them.
+constexpr int SA_PV = 4;      // value rows in flight per step
+
+template <typename T, int DPL, int REP>
 __global__ void __launch_bounds__(SA_WAVES * WAVE)
 sink_attn_kernel(const T* __restrict__ q, long q_tok,
                  const T* __restrict__ k_cache, const T* __restrict__ v_cache,
@@ -829,78 +884,105 @@ sink_attn_kernel(const T* __restrict__ q, long q_tok,
                  long out_tok, float out_scale, float* __restrict__ part_acc,
                  float* __restrict__ part_ml, int Tn, int H, int G, int D,
                  int Dv, int bs, int window) {
-    __shared__ float qs[SA_WAVES][SA_MAXD];
+    extern __shared__ __attribute__((aligned(16))) float sa_q[];
     const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-    const int t = blockIdx.x, h = blockIdx.y * SA_WAVES + wid;
-    if (h >= H) return;      // no workgroup barrier below
+    const int t = blockIdx.x;
+    const int unit = blockIdx.y * SA_WAVES + wid;   // REP consecutive heads
+    if (unit * REP >= H) return;      // no workgroup barrier below
+    const int h0 = unit * REP;
     const int split = blockIdx.z, nsplit = gridDim.z;
     const int p = positions[t];
-    const int g = h / (H / G);
+    const int g = h0 / (H / G);
     const int lo = window > 0 ? max(0, p - window + 1) : 0;
     const int per = (p + 1 - lo + nsplit - 1) / nsplit;
     const int klo = lo + split * per, khi = min(p + 1, klo + per);
-    float* qv = qs[wid];
-    for (int i = lane; i < D; i += WAVE)
-        qv[i] = ldf(q + (long)t * q_tok + (long)h * D + i);
+    float* qv = sa_q + (long)wid * REP * D;
+    for (int i = lane; i < REP * D; i += WAVE)
+        qv[i] = ldf(q + (long)t * q_tok + (long)h0 * D + i);
     WAVE_LDS_SYNC();
     const int* bt = block_table + (long)seq_idx[t] * bt_stride;
-    float m = -INFINITY, l = 0.f;
-    float acc[DPL];
+    float m[REP], l[REP], acc[REP][DPL];
 #pragma unroll
-    for (int i = 0; i < DPL; ++i) acc[i] = 0.f;
+    for (int r = 0; r < REP; ++r) {
+        m[r] = -INFINITY;
+        l[r] = 0.f;
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) acc[r][i] = 0.f;
+    }
     for (int j0 = klo; j0 < khi; j0 += WAVE) {
         const int j = j0 + lane;
         const bool valid = j < khi;
-        int row = 0;
-        float sc = -INFINITY;
+        int row = 0;            // lanes past the end point at a real row
+        float sc[REP], pj[REP];
+#pragma unroll
+        for (int r = 0; r < REP; ++r) sc[r] = 0.f;
         if (valid) {
             row = (bt[j / bs] * G + g) * bs + j % bs;
-            sc = sa_dot<T>(k_cache + (long)row * D, qv, D);
+            SaDots<T, REP>::run(k_cache + (long)row * D, qv, D, sc);
         }
-        const float m_new = fmaxf(m, wave_max(sc));
-        const float pj = valid ? expf(sc - m_new) : 0.f;
-        const float corr = expf(m - m_new);
-        l = l * corr + wave_sum(pj);
 #pragma unroll
-        for (int i = 0; i < DPL; ++i) acc[i] *= corr;
+        for (int r = 0; r < REP; ++r) {
+            const float s = valid ? sc[r] : -INFINITY;
+            const float m_new = fmaxf(m[r], wave_max(s));
+            pj[r] = valid ? expf(s - m_new) : 0.f;
+            const float corr = expf(m[r] - m_new);
+            l[r] = l[r] * corr + wave_sum(pj[r]);
+#pragma unroll
+            for (int i = 0; i < DPL; ++i) acc[r][i] *= corr;
+            m[r] = m_new;
+        }
         const int nk = min(WAVE, khi - j0);
-        for (int jj = 0; jj < nk; ++jj) {
-            const float pb = __shfl(pj, jj);
-            const T* vr = v_cache + (long)__shfl(row, jj) * Dv;
+        for (int jj = 0; jj < nk; jj += SA_PV) {
+            float vv[SA_PV][DPL];
+#pragma unroll
+            for (int u = 0; u < SA_PV; ++u) {
+                const T* vr = v_cache + (long)__shfl(row, jj + u) * Dv;
+#pragma unroll
+                for (int i = 0; i < DPL; ++i) {
+                    const int d = lane + i * WAVE;
+                    vv[u][i] = d < Dv ? ldf(vr + d) : 0.f;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < SA_PV; ++u)
+#pragma unroll
+                for (int r = 0; r < REP; ++r) {
+                    const float pb = __shfl(pj[r], jj + u);
+#pragma unroll
+                    for (int i = 0; i < DPL; ++i) acc[r][i] += pb * vv[u][i];
+                }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < REP; ++r) {
+        const int h = h0 + r;
+        if (nsplit == 1) {
+            float L = l[r], w = 1.f;
+            if (sink) {
+                const float sk = sink[h];
+                const float M = fmaxf(m[r], sk);
+                w = expf(m[r] - M);
+                L = l[r] * w + expf(sk - M);
+            }
+            const float rcp = L > 0.f ? out_scale * w / L : 0.f;
+            T* o = out + (long)t * out_tok + (long)h * Dv;
 #pragma unroll
             for (int i = 0; i < DPL; ++i) {
                 const int d = lane + i * WAVE;
-                if (d < Dv) acc[i] += pb * ldf(vr + d);
+                if (d < Dv) stf(o + d, acc[r][i] * rcp);
+            }
+        } else {
+            const long prow = ((long)split * H + h) * Tn + t;
+            if (lane == 0) {
+                part_ml[prow * 2] = m[r];
+                part_ml[prow * 2 + 1] = l[r];
+            }
+#pragma unroll
+            for (int i = 0; i < DPL; ++i) {
+                const int d = lane + i * WAVE;
+                if (d < Dv) part_acc[prow * Dv + d] = acc[r][i];
             }
         }
-        m = m_new;
-    }
-    if (nsplit == 1) {
-        float L = l, w = 1.f;
-        if (sink) {
-            const float sk = sink[h];
-            const float M = fmaxf(m, sk);
-            w = expf(m - M);
-            L = l * w + expf(sk - M);
-        }
-        const float rcp = L > 0.f ? out_scale * w / L : 0.f;
-        T* o = out + (long)t * out_tok + (long)h * Dv;
-#pragma unroll
-        for (int i = 0; i < DPL; ++i) {
-            const int d = lane + i * WAVE;
-            if (d < Dv) stf(o + d, acc[i] * rcp);
-        }
-        return;
-    }
-    const long prow = ((long)split * H + h) * Tn + t;
-    if (lane == 0) {
-        part_ml[prow * 2] = m;
-        part_ml[prow * 2 + 1] = l;
-    }
-#pragma unroll
-    for (int i = 0; i < DPL; ++i) {
-        const int d = lane + i * WAVE;
-        if (d < Dv) part_acc[prow * Dv + d] = acc[i];
     }
 }
 
@@ -1153,13 +1235,17 @@ extern "C" int launch_delta_rule(const float* q, const float* k, long qk_tok,
     return 0;
 }
 
+#define SA_LAUNCH(N, R)                                                       \
+    sink_attn_kernel<TT, N, R><<<grid, SA_WAVES * WAVE, smem, s>>>(           \
+        (const TT*)q, q_tok, (const TT*)k_cache, (const TT*)v_cache,          \
+        block_table, bt_stride, positions, seq_idx, sink, (TT*)out, out_tok,  \
+        out_scale, part_acc, part_ml, Tn, H, G, D, Dv, bs, window)
+
 #define SA_CASE(N)                                                            \
     case N:                                                                   \
-        sink_attn_kernel<TT, N><<<grid, SA_WAVES * WAVE, 0, s>>>(             \
-            (const TT*)q, q_tok, (const TT*)k_cache, (const TT*)v_cache,      \
-            block_table, bt_stride, positions, seq_idx, sink, (TT*)out,       \
-            out_tok, out_scale, part_acc, part_ml, Tn, H, G, D, Dv, bs,       \
-            window);                                                          \
+        if (rep == 4) SA_LAUNCH(N, 4);                                        \
+        else if (rep == 2) SA_LAUNCH(N, 2);                                   \
+        else SA_LAUNCH(N, 1);                                                 \
         break;
 
 template <typename TT>
@@ -1172,7 +1258,12 @@ static int sink_attn_dispatch(const void* q, long q_tok, const void* k_cache,
                               int Tn, int H, int G, int D, int Dv, int bs,
                               int window, hipStream_t s) {
     const int dpl = (Dv + WAVE - 1) / WAVE;
-    const dim3 grid(Tn, (H + SA_WAVES - 1) / SA_WAVES, splits);
+    // query heads per wave: the largest of 4, 2, 1 that divides the group
+    const int group = H / G;
+    const int rep = group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
+    const int units = H / rep;
+    const dim3 grid(Tn, (units + SA_WAVES - 1) / SA_WAVES, splits);
+    const size_t smem = (size_t)SA_WAVES * rep * D * sizeof(float);
     switch (dpl) {
         SA_CASE(1) SA_CASE(2) SA_CASE(3) SA_CASE(4)
         default: return 1;

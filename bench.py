@@ -40,7 +40,6 @@ def compare_hybrid(args) -> None:
     closest dense-attention stack the framework serves (GQA attention,
     routed experts) at the same width, depth and expert sizes. Random
     weights, synthetic prompts, one GPU."""
-    from bee2bee_amd.engine.engine import InferenceEngine
     from bee2bee_amd.models.hybrid import nukopel_layers
     from bee2bee_amd.models.spec import ModelSpec, hybrid_spec
 
@@ -49,12 +48,6 @@ def compare_hybrid(args) -> None:
     vocab, head_dim = 32000, 128
     p_batch, p_len = 8, (2048 if on_gpu else 64)
     d_batch, d_len = (64 if on_gpu else 4), (1024 if on_gpu else 32)
-    budget = args.warmup + args.steps + 4
-
-    def sync() -> None:
-        if on_gpu:
-            torch.cuda.synchronize()
-
     for size in args.compare_hybrid.split(","):
         z = HYBRID_SIZES[size.strip()]
         W, H, L = z["width"], z["heads"], z["layers"]
@@ -72,46 +65,112 @@ def compare_hybrid(args) -> None:
             n_kv_heads=max(1, H // 4), head_dim=head_dim, rope_theta=1e6,
             max_seq_len=8192, n_experts=z["experts"], top_k_experts=2)
         for spec in (nk, dense):
-            engine = InferenceEngine(
-                spec, device=device, max_batch=max(d_batch, p_batch),
-                max_seq_len=max(p_len, d_len) + budget + 8,
-                use_graphs=(not args.no_graphs) and on_gpu,
-                max_prefill_tokens=8192, seed=1234)
-            times = []
-            for _ in range(2):           # first pass is the warmup
-                sync()
-                t0 = time.perf_counter()
-                ids = engine.bench_prefill(p_batch, p_len, max_new=1)
-                sync()
-                times.append(time.perf_counter() - t0)
-                for sid in ids:
-                    engine.kv.free_seq(sid)
-            prefill_tps = p_batch * p_len / times[-1]
-            engine.bench_setup(d_batch, d_len, budget)
-            for _ in range(args.warmup):
-                engine.bench_step()
-            sync()
-            t0 = time.perf_counter()
-            for _ in range(args.steps):
-                engine.bench_step()
-            sync()
-            dt = time.perf_counter() - t0
-            print(json.dumps({
-                "compare": "hybrid-vs-dense", "size": size, "model": spec.name,
-                "params_m": round(spec.n_params() / 1e6, 1),
-                "prefill_tokens_per_s": round(prefill_tps, 1),
-                "prefill_shape": [p_batch, p_len],
-                "decode_tokens_per_s": round(d_batch * args.steps / dt, 1),
-                "decode_ms_per_step": round(dt / args.steps * 1e3, 3),
-                "decode_shape": [d_batch, d_len],
-                "decode_graphs": engine.graphs is not None,
-                "dtype": "bf16" if on_gpu else "fp32-cpu",
-                "data": "synthetic",
-            }), flush=True)
-            engine.shutdown()
-            del engine
-            if on_gpu:
-                torch.cuda.empty_cache()
+            _measure_prefill_decode(spec, "hybrid-vs-dense", size, args,
+                                    device, p_batch, p_len, d_batch, d_len)
+
+
+def _measure_prefill_decode(spec, label, size, args, device, p_batch, p_len,
+                            d_batch, d_len) -> None:
+    """One JSON line: prefill tokens/s of p_batch prompts of p_len tokens in
+    one step, and decode tokens/s of d_batch sequences at context d_len."""
+    from bee2bee_amd.engine.engine import InferenceEngine
+
+    on_gpu = device != "cpu"
+    budget = args.warmup + args.steps + 4
+
+    def sync() -> None:
+        if on_gpu:
+            torch.cuda.synchronize()
+
+    engine = InferenceEngine(
+        spec, device=device, max_batch=max(d_batch, p_batch),
+        max_seq_len=max(p_len, d_len) + budget + 8,
+        use_graphs=(not args.no_graphs) and on_gpu,
+        max_prefill_tokens=p_batch * p_len, seed=1234)
+    times = []
+    for _ in range(2):           # first pass is the warmup
+        sync()
+        t0 = time.perf_counter()
+        ids = engine.bench_prefill(p_batch, p_len, max_new=1)
+        sync()
+        times.append(time.perf_counter() - t0)
+        for sid in ids:
+            engine.kv.free_seq(sid)
+    prefill_tps = p_batch * p_len / times[-1]
+    engine.bench_setup(d_batch, d_len, budget)
+    for _ in range(args.warmup):
+        engine.bench_step()
+    sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        engine.bench_step()
+    sync()
+    dt = time.perf_counter() - t0
+    print(json.dumps({
+        "compare": label, "size": size, "model": spec.name,
+        "params_m": round(spec.n_params() / 1e6, 1),
+        "prefill_tokens_per_s": round(prefill_tps, 1),
+        "prefill_shape": [p_batch, p_len],
+        "decode_tokens_per_s": round(d_batch * args.steps / dt, 1),
+        "decode_ms_per_step": round(dt / args.steps * 1e3, 3),
+        "decode_shape": [d_batch, d_len],
+        "decode_graphs": engine.graphs is not None,
+        "dtype": "bf16" if on_gpu else "fp32-cpu",
+        "data": "synthetic",
+    }), flush=True)
+    engine.shutdown()
+    del engine
+    if on_gpu:
+        torch.cuda.empty_cache()
+
+
+# layer sizes for --compare-pugozen: (width, heads, layers, ff of relu^2 MLP)
+PUGOZEN_SIZES = {
+    "s": dict(width=1024, heads=8, layers=6, ff=4096),
+    "m": dict(width=2048, heads=16, layers=6, ff=8192),
+    "l": dict(width=4096, heads=32, layers=6, ff=16384),
+}
+
+
+def compare_pugozen(args) -> None:
+    """Prefill and decode throughput of a Pugozen stack (the cycle
+    attention+delta / retention / delta, dense relu^2 feed-forward, fused
+    per-layer input and output GEMMs) beside the closest stack the framework
+    already served: a dense GQA transformer of equal width, depth, head
+    count/size and feed-forward parameter count. Random weights, synthetic
+    prompts, one GPU."""
+    from bee2bee_amd.models.hybrid import pugozen_layers
+    from bee2bee_amd.models.spec import ModelSpec, hybrid_spec
+
+    on_gpu = torch.cuda.is_available()
+    device = "cuda:0" if on_gpu else "cpu"
+    vocab, head_dim = 32000, 128
+    p_batch, p_len = 8, (2048 if on_gpu else 48)
+    d_batch, d_len = (64 if on_gpu else 4), (1024 if on_gpu else 32)
+    for size in args.compare_pugozen.split(","):
+        z = PUGOZEN_SIZES[size.strip()]
+        W, H, L = z["width"], z["heads"], z["layers"]
+        if not on_gpu:
+            W, H, L, head_dim, vocab = 64, 2, 3, 16, 256
+            z = dict(z, ff=128)
+        pz = hybrid_spec(
+            f"pugozen-{size}", vocab, W,
+            pugozen_layers(L, W, heads=H, kv_heads=max(1, H // 4),
+                           dim=head_dim, ff=z["ff"], delta_heads=H,
+                           delta_kv_heads=max(1, H // 2), delta_dim=head_dim,
+                           rank=64 if on_gpu else 8,
+                           side_heads=max(1, H // 4), side_dim=head_dim // 2),
+            eps=1e-6, embed_scale=1.0, canon_taps=0, max_seq_len=8192,
+            arch="pugozen", norm_type="rmsnorm", act_type="relu2")
+        dense = ModelSpec(
+            name=f"gqa-dense-{size}", vocab_size=vocab, hidden_size=W,
+            # a gated MLP has three matrices: equal parameters at 2/3 ff
+            intermediate_size=z["ff"] * 2 // 3 // 64 * 64, n_layers=L,
+            n_heads=H, n_kv_heads=max(1, H // 4), head_dim=head_dim,
+            rope_theta=1e6, max_seq_len=8192)
+        for spec in (pz, dense):
+            _measure_prefill_decode(spec, "pugozen-vs-dense", size, args,
+                                    device, p_batch, p_len, d_batch, d_len)
 
 
 def main() -> None:
@@ -134,6 +193,13 @@ def main() -> None:
                          "dense-attention MoE stack of equal width, depth "
                          "and expert sizes, at the comma-separated sizes "
                          "(s, m, l); one JSON line per size and model")
+    ap.add_argument("--compare-pugozen", default=None, metavar="SIZES",
+                    help="instead of the headline run: prefill and decode "
+                         "throughput of the Pugozen stack (attention+delta / "
+                         "retention / delta layers, relu^2 feed-forward) "
+                         "beside a dense GQA transformer of equal width, "
+                         "depth and heads, at the comma-separated sizes "
+                         "(s, m, l); one JSON line per size and model")
     ap.add_argument("--preflight", action="store_true",
                     help="run the scale-run preflight checks (RCCL self-"
                          "test, master endpoint, env, rank wiring) and exit")
@@ -150,6 +216,9 @@ def main() -> None:
 
     if args.compare_hybrid:
         compare_hybrid(args)
+        return
+    if args.compare_pugozen:
+        compare_pugozen(args)
         return
 
     from bee2bee_amd.models.spec import resolve_spec
