@@ -693,11 +693,14 @@ void sink_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache,
                              "its guard admitted");
         return;
     }
-    // few rows (decode): split each row's keys over more workgroups, at
-    // least 128 keys per share of the longest context the tables can hold
+    // few rows (decode): split each row's keys over more waves, at least 64
+    // keys per share of the longest context the tables can hold
     const long ctx = window > 0 ? window : block_table.size(1) * (long)bs;
-    long splits = 8192 / std::max<long>(1, (long)Tn * H);
-    splits = std::min<long>({splits, 16, (ctx + 127) / 128});
+    // a wave serves up to 4 query heads of one key group (mixers.hip)
+    const long group = H / G;
+    const long units = H / (group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1);
+    long splits = 8192 / std::max<long>(1, (long)Tn * units);
+    splits = std::min<long>({splits, 32, (ctx + 63) / 64});
     splits = std::max<long>(splits, 1);
     Tensor part_acc, part_ml;
     float *pa = nullptr, *pm = nullptr;

@@ -652,18 +652,33 @@ __global__ void lightning_scan_kernel(const float* __restrict__ decay,
 // token:  M <- g * M;  delta = beta (v - M^T k);  M <- M + k delta^T;
 // y = M^T q.  Since y = (gM)^T q + delta (k . q), both sums over the key
 // axis run on the faded memory in ONE pass.
-// A workgroup is ONE wave that owns DR_CW columns of one (sequence, value
-// head) state: lane (r, c) keeps rows [r*DPT, (r+1)*DPT) of column c in
-// registers, the DR_RG row groups are combined with two xor-shuffles, and
-// nothing but the staging of DR_TB tokens' q/k/g/v/beta through LDS needs a
-// barrier. Columns evolve independently -> sequences x heads x Dv/DR_CW
-// waves. Tokens are walked in order (the update of token t reads the state
-// token t-1 left).
-constexpr int DR_RG = 4;
-constexpr int DR_CW = WAVE / DR_RG;
+// A workgroup is ONE wave that owns 64/RG columns of one (sequence, value
+// head) state: lane (c, r) = (lane / RG, lane % RG) keeps rows
+// [r*DPT, (r+1)*DPT) of column c in registers. The RG row groups are
+// neighbouring lanes, so the two sums over the key axis are DPP adds inside
+// a row of 16 lanes (no LDS round trip), and nothing but the staging of
+// DR_TB tokens' q/k/g/v/beta through LDS needs a barrier. Columns evolve
+// independently -> sequences x heads x Dv*RG/64 waves; the launcher picks
+// RG = 4 when sequences x heads alone fill the chip (decode: 64-byte state
+// rows per group) and 8 or 16 for a few long prompt portions. Tokens are
+// walked in order (token t reads the state token t-1 left).
 constexpr int DR_TB = 8;
 
-template <int DPT, bool CHDEC>
+template <int CTRL> DEV_INLINE float dr_dpp_add(float x) {
+    const int y = __builtin_amdgcn_update_dpp(
+        0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true);
+    return x + __builtin_bit_cast(float, y);
+}
+// sum over the RG neighbouring lanes of a group; every lane gets the total
+template <int RG> DEV_INLINE float dr_group_sum(float x) {
+    x = dr_dpp_add<0xB1>(x);                  // quad_perm [1,0,3,2]
+    x = dr_dpp_add<0x4E>(x);                  // quad_perm [2,3,0,1]
+    if (RG >= 8) x = dr_dpp_add<0x141>(x);    // row_half_mirror
+    if (RG >= 16) x = dr_dpp_add<0x140>(x);   // row_mirror
+    return x;
+}
+
+template <int DPT, int RG, bool CHDEC>
 __global__ void __launch_bounds__(WAVE)
 delta_rule_kernel(const float* __restrict__ q, const float* __restrict__ k,
                   long qk_tok, const float* __restrict__ v, long v_tok,
@@ -675,18 +690,21 @@ delta_rule_kernel(const float* __restrict__ q, const float* __restrict__ k,
                   const int* __restrict__ positions,
                   float* __restrict__ out,          // [Tn, H, Dv]
                   int H, int G, int D, int Dv) {
-    constexpr int DMAX = DPT * DR_RG;
+    static_assert(DPT % 4 == 0, "16-byte LDS reads");
+    constexpr int DMAX = DPT * RG;
+    constexpr int CW = WAVE / RG;
     __shared__ __attribute__((aligned(16))) float qs[DR_TB][DMAX];
     __shared__ __attribute__((aligned(16))) float ks[DR_TB][DMAX];
     __shared__ __attribute__((aligned(16))) float gs[DR_TB][CHDEC ? DMAX : 4];
-    __shared__ float vs[DR_TB][DR_CW];
+    __shared__ float vs[DR_TB][CW];
     __shared__ float bs[DR_TB];
+    __shared__ float kqs[DR_TB];
     const int b = blockIdx.x, h = blockIdx.y;
     const int lo = cu[b], hi = cu[b + 1];
     if (hi <= lo) return;
     const int lane = threadIdx.x;
-    const int r = lane / DR_CW, c = lane % DR_CW;
-    const int c0 = blockIdx.z * DR_CW;
+    const int c = lane / RG, r = lane % RG;
+    const int c0 = blockIdx.z * CW;
     const int dv = c0 + c;
     const bool live = dv < Dv;
     const int d0 = r * DPT;
@@ -709,8 +727,8 @@ delta_rule_kernel(const float* __restrict__ q, const float* __restrict__ k,
             if (CHDEC)
                 gs[tt][d] = d < D ? g[((long)(t0 + tt) * H + h) * D + d] : 1.f;
         }
-        for (int idx = lane; idx < n * DR_CW; idx += WAVE) {
-            const int tt = idx / DR_CW, cc = idx - tt * DR_CW;
+        for (int idx = lane; idx < n * CW; idx += WAVE) {
+            const int tt = idx / CW, cc = idx - tt * CW;
             vs[tt][cc] = (c0 + cc < Dv)
                 ? v[(long)(t0 + tt) * v_tok + (long)h * Dv + c0 + cc] : 0.f;
         }
@@ -719,39 +737,38 @@ delta_rule_kernel(const float* __restrict__ q, const float* __restrict__ k,
             if (!CHDEC) gs[lane][0] = g[(long)(t0 + lane) * H + h];
         }
         __syncthreads();
+        // k . q of each staged token, once (it does not involve the state)
+        for (int tt = 0; tt < n; ++tt) {
+            float a = 0.f;
+            for (int d = lane; d < DMAX; d += WAVE) a += ks[tt][d] * qs[tt][d];
+            a = wave_sum(a);
+            if (lane == 0) kqs[tt] = a;
+        }
+        __syncthreads();
         for (int tt = 0; tt < n; ++tt) {
             // this lane's slice of k, q (and the per-channel decay) into
             // registers with 16-byte LDS reads; k is used twice
             float kr[DPT], qr[DPT], gr[CHDEC ? DPT : 1];
-            if constexpr (DPT % 4 == 0) {
 #pragma unroll
-                for (int i = 0; i < DPT; i += 4) {
-                    const f32x4 a =
-                        *reinterpret_cast<const f32x4*>(&ks[tt][d0 + i]);
-                    const f32x4 b =
-                        *reinterpret_cast<const f32x4*>(&qs[tt][d0 + i]);
+            for (int i = 0; i < DPT; i += 4) {
+                const f32x4 a =
+                    *reinterpret_cast<const f32x4*>(&ks[tt][d0 + i]);
+                const f32x4 e =
+                    *reinterpret_cast<const f32x4*>(&qs[tt][d0 + i]);
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        kr[i + j] = a[j];
-                        qr[i + j] = b[j];
-                    }
-                    if constexpr (CHDEC) {
-                        const f32x4 e =
-                            *reinterpret_cast<const f32x4*>(&gs[tt][d0 + i]);
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) gr[i + j] = e[j];
-                    }
+                for (int j = 0; j < 4; ++j) {
+                    kr[i + j] = a[j];
+                    qr[i + j] = e[j];
                 }
-            } else {
+                if constexpr (CHDEC) {
+                    const f32x4 w =
+                        *reinterpret_cast<const f32x4*>(&gs[tt][d0 + i]);
 #pragma unroll
-                for (int i = 0; i < DPT; ++i) {
-                    kr[i] = ks[tt][d0 + i];
-                    qr[i] = qs[tt][d0 + i];
-                    if constexpr (CHDEC) gr[i] = gs[tt][d0 + i];
+                    for (int j = 0; j < 4; ++j) gr[i + j] = w[j];
                 }
             }
             if constexpr (!CHDEC) gr[0] = gs[tt][0];
-            float ka = 0.f, kb = 0.f, qa = 0.f, qb = 0.f, kq = 0.f;
+            float ka = 0.f, kb = 0.f, qa = 0.f, qb = 0.f;
 #pragma unroll
             for (int i = 0; i < DPT; i += 2) {
                 const float s0 = s[i] * gr[CHDEC ? i : 0];
@@ -762,20 +779,14 @@ delta_rule_kernel(const float* __restrict__ q, const float* __restrict__ k,
                 kb += kr[i + 1] * s1;
                 qa += qr[i] * s0;
                 qb += qr[i + 1] * s1;
-                kq += kr[i] * qr[i] + kr[i + 1] * qr[i + 1];
             }
-            float kS = ka + kb, qS = qa + qb;
-#pragma unroll
-            for (int off = DR_CW; off < WAVE; off <<= 1) {
-                kS += __shfl_xor(kS, off);
-                qS += __shfl_xor(qS, off);
-                kq += __shfl_xor(kq, off);
-            }
+            const float kS = dr_group_sum<RG>(ka + kb);
+            const float qS = dr_group_sum<RG>(qa + qb);
             const float u = bs[tt] * (vs[tt][c] - kS);
 #pragma unroll
             for (int i = 0; i < DPT; ++i) s[i] += kr[i] * u;
             if (r == 0 && live)
-                out[((long)(t0 + tt) * H + h) * Dv + dv] = qS + u * kq;
+                out[((long)(t0 + tt) * H + h) * Dv + dv] = qS + u * kqs[tt];
         }
         __syncthreads();
     }
@@ -871,7 +882,7 @@ template <int REP> struct SaDots<unsigned short, REP> {
 
 // A wave serves REP query heads that share one key/value head (REP divides
 // the group size), so each cached row is read once for all of them.
-constexpr int SA_PV = 4;      // value rows in flight per step
+constexpr int SA_PV = 8;      // value rows in flight per step
 
 template <typename T, int DPL, int REP>
 __global__ void __launch_bounds__(SA_WAVES * WAVE)
@@ -1201,17 +1212,21 @@ extern "C" int launch_lightning(const void* q, const void* k, const void* v,
 #undef LI_DISPATCH
 }
 
-#define DR_CASE(N)                                                            \
-    case N:                                                                   \
+#define DR_LAUNCH(N, R)                                                       \
+    do {                                                                      \
+        const dim3 grid(B, H, (Dv * R + WAVE - 1) / WAVE);                    \
         if (chdec)                                                            \
-            delta_rule_kernel<N, true><<<grid, WAVE, 0, s>>>(                 \
+            delta_rule_kernel<N, R, true><<<grid, WAVE, 0, s>>>(              \
                 q, k, qk_tok, v, v_tok, beta, g, state, state_slots, cu,      \
                 positions, out, H, G, D, Dv);                                 \
         else                                                                  \
-            delta_rule_kernel<N, false><<<grid, WAVE, 0, s>>>(                \
+            delta_rule_kernel<N, R, false><<<grid, WAVE, 0, s>>>(             \
                 q, k, qk_tok, v, v_tok, beta, g, state, state_slots, cu,      \
                 positions, out, H, G, D, Dv);                                 \
-        break;
+    } while (0)
+
+#define DR_CASE(N, R)                                                         \
+    if (rg == R && dpt == N) { DR_LAUNCH(N, R); return 0; }
 
 // returns nonzero when the key dim exceeds 256
 extern "C" int launch_delta_rule(const float* q, const float* k, long qk_tok,
@@ -1222,17 +1237,19 @@ extern "C" int launch_delta_rule(const float* q, const float* k, long qk_tok,
                                  float* out, int B, int H, int G, int D,
                                  int Dv, hipStream_t s) {
     if (B == 0) return 0;
-    const int need = (D + DR_RG - 1) / DR_RG;
-    const int sizes[] = {2, 4, 8, 16, 32, 64};
-    int dpt = 0;
-    for (int z : sizes)
-        if (z >= need) { dpt = z; break; }
-    if (!dpt) return 1;
-    const dim3 grid(B, H, (Dv + DR_CW - 1) / DR_CW);
-    switch (dpt) {
-        DR_CASE(2) DR_CASE(4) DR_CASE(8) DR_CASE(16) DR_CASE(32) DR_CASE(64)
-    }
-    return 0;
+    if (D > 256) return 1;
+    // row groups per column: 4 unless that leaves the chip short of about
+    // two waves per SIMD (a few long portions), then 8 or 16
+    int rg = 4;
+    while (rg < 16 && (long)B * H * ((Dv * rg + WAVE - 1) / WAVE) < 2048)
+        rg <<= 1;
+    const int need = (D + rg - 1) / rg;
+    const int dpt = need <= 4 ? 4 : need <= 8 ? 8 : need <= 16 ? 16
+                    : need <= 32 ? 32 : 64;
+    DR_CASE(4, 4) DR_CASE(8, 4) DR_CASE(16, 4) DR_CASE(32, 4) DR_CASE(64, 4)
+    DR_CASE(4, 8) DR_CASE(8, 8) DR_CASE(16, 8) DR_CASE(32, 8)
+    DR_CASE(4, 16) DR_CASE(8, 16) DR_CASE(16, 16)
+    return 1;
 }
 
 #define SA_LAUNCH(N, R)                                                       \

@@ -101,7 +101,9 @@ def test_delta_gates(dtype, G, H, D, chan):
 
 @pytest.mark.parametrize("G,H,D,Dv,chan", [
     (2, 4, 24, 40, False), (3, 3, 40, 24, True), (1, 2, 64, 64, True),
-    (2, 2, 128, 128, False), (1, 1, 7, 5, True), (2, 4, 200, 20, False)])
+    (2, 2, 128, 128, False), (1, 1, 7, 5, True), (2, 4, 200, 20, False),
+    # enough (sequence, head, column) work for 8 and for 4 row groups
+    (8, 32, 16, 128, True), (64, 64, 12, 128, False)])
 def test_delta_rule(G, H, D, Dv, chan):
     torch.manual_seed(4)
     m = batch_meta([19, 1, 2, 33], [0, 7, 1, 3], 16, 8)
