@@ -717,32 +717,68 @@ delta_rule_kernel(const float* __restrict__ q, const float* __restrict__ k,
         const int d = d0 + i;
         s[i] = (!fresh && live && d < D) ? st[(long)d * Dv] : 0.f;
     }
-    for (int t0 = lo; t0 < hi; t0 += DR_TB) {
+    // The next DR_TB tokens' inputs are fetched into registers while the
+    // current ones are consumed from LDS, so HBM latency stays off the
+    // token-serial chain.
+    constexpr int PQ = (DR_TB * DMAX + WAVE - 1) / WAVE;
+    constexpr int PV = (DR_TB * CW + WAVE - 1) / WAVE;
+    float pq[PQ], pk[PQ], pg[CHDEC ? PQ : 1], pv[PV], pb = 0.f;
+    auto fetch = [&](int t0) {
         const int n = min(DR_TB, hi - t0);
-        for (int idx = lane; idx < n * DMAX; idx += WAVE) {
+#pragma unroll
+        for (int e = 0; e < PQ; ++e) {
+            const int idx = lane + e * WAVE;
             const int tt = idx / DMAX, d = idx - tt * DMAX;
+            const bool ok = tt < n && d < D;
             const long base = (long)(t0 + tt) * qk_tok + (long)kvh * D + d;
-            qs[tt][d] = d < D ? q[base] : 0.f;
-            ks[tt][d] = d < D ? k[base] : 0.f;
+            pq[e] = ok ? q[base] : 0.f;
+            pk[e] = ok ? k[base] : 0.f;
             if (CHDEC)
-                gs[tt][d] = d < D ? g[((long)(t0 + tt) * H + h) * D + d] : 1.f;
+                pg[e] = ok ? g[((long)(t0 + tt) * H + h) * D + d] : 1.f;
         }
-        for (int idx = lane; idx < n * CW; idx += WAVE) {
+#pragma unroll
+        for (int e = 0; e < PV; ++e) {
+            const int idx = lane + e * WAVE;
             const int tt = idx / CW, cc = idx - tt * CW;
-            vs[tt][cc] = (c0 + cc < Dv)
+            pv[e] = (tt < n && c0 + cc < Dv)
                 ? v[(long)(t0 + tt) * v_tok + (long)h * Dv + c0 + cc] : 0.f;
         }
         if (lane < n) {
-            bs[lane] = beta[(long)(t0 + lane) * H + h];
-            if (!CHDEC) gs[lane][0] = g[(long)(t0 + lane) * H + h];
+            pb = beta[(long)(t0 + lane) * H + h];
+            if (!CHDEC) pg[0] = g[(long)(t0 + lane) * H + h];
+        }
+    };
+    fetch(lo);
+    for (int t0 = lo; t0 < hi; t0 += DR_TB) {
+        const int n = min(DR_TB, hi - t0);
+#pragma unroll
+        for (int e = 0; e < PQ; ++e) {
+            const int idx = lane + e * WAVE;
+            if (idx < DR_TB * DMAX) {
+                (&qs[0][0])[idx] = pq[e];
+                (&ks[0][0])[idx] = pk[e];
+                if (CHDEC) (&gs[0][0])[idx] = pg[e];
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < PV; ++e) {
+            const int idx = lane + e * WAVE;
+            if (idx < DR_TB * CW) (&vs[0][0])[idx] = pv[e];
+        }
+        if (lane < n) {
+            bs[lane] = pb;
+            if (!CHDEC) gs[lane][0] = pg[0];
         }
         __syncthreads();
-        // k . q of each staged token, once (it does not involve the state)
-        for (int tt = 0; tt < n; ++tt) {
+        if (t0 + DR_TB < hi) fetch(t0 + DR_TB);
+        // k . q of each staged token, once (it does not involve the state):
+        // 8 neighbouring lanes per token
+        {
+            const int tt = lane / 8, part = lane % 8;
             float a = 0.f;
-            for (int d = lane; d < DMAX; d += WAVE) a += ks[tt][d] * qs[tt][d];
-            a = wave_sum(a);
-            if (lane == 0) kqs[tt] = a;
+            for (int d = part; d < DMAX; d += 8) a += ks[tt][d] * qs[tt][d];
+            a = dr_group_sum<8>(a);
+            if (part == 0) kqs[tt] = a;
         }
         __syncthreads();
         for (int tt = 0; tt < n; ++tt) {
@@ -927,10 +963,9 @@ sink_attn_kernel(const T* __restrict__ q, long q_tok,
         float sc[REP], pj[REP];
 #pragma unroll
         for (int r = 0; r < REP; ++r) sc[r] = 0.f;
-        if (valid) {
-            row = (bt[j / bs] * G + g) * bs + j % bs;
-            SaDots<T, REP>::run(k_cache + (long)row * D, qv, D, sc);
-        }
+        const int nk = min(WAVE, khi - j0);
+        if (valid) row = (bt[j / bs] * G + g) * bs + j % bs;
+        if (valid) SaDots<T, REP>::run(k_cache + (long)row * D, qv, D, sc);
 #pragma unroll
         for (int r = 0; r < REP; ++r) {
             const float s = valid ? sc[r] : -INFINITY;
@@ -942,12 +977,13 @@ sink_attn_kernel(const T* __restrict__ q, long q_tok,
             for (int i = 0; i < DPL; ++i) acc[r][i] *= corr;
             m[r] = m_new;
         }
-        const int nk = min(WAVE, khi - j0);
+#pragma unroll 2
         for (int jj = 0; jj < nk; jj += SA_PV) {
             float vv[SA_PV][DPL];
 #pragma unroll
             for (int u = 0; u < SA_PV; ++u) {
-                const T* vr = v_cache + (long)__shfl(row, jj + u) * Dv;
+                const T* vr =
+                    v_cache + (long)__builtin_amdgcn_readlane(row, jj + u) * Dv;
 #pragma unroll
                 for (int i = 0; i < DPL; ++i) {
                     const int d = lane + i * WAVE;
@@ -958,7 +994,10 @@ sink_attn_kernel(const T* __restrict__ q, long q_tok,
             for (int u = 0; u < SA_PV; ++u)
 #pragma unroll
                 for (int r = 0; r < REP; ++r) {
-                    const float pb = __shfl(pj[r], jj + u);
+                    // jj + u is wave-uniform: a scalar lane read, no LDS trip
+                    const float pb = __builtin_bit_cast(
+                        float, __builtin_amdgcn_readlane(
+                                   __builtin_bit_cast(int, pj[r]), jj + u));
 #pragma unroll
                     for (int i = 0; i < DPL; ++i) acc[r][i] += pb * vv[u][i];
                 }
@@ -1023,12 +1062,21 @@ sink_attn_combine_kernel(const float* __restrict__ part_acc,
     T* o = out + (long)t * out_tok + (long)h * Dv;
     for (int d0 = 0; d0 < Dv; d0 += WAVE) {
         const int d = d0 + lane;
+        const int dc = min(d, Dv - 1);      // clamped: every load is valid
         float a = 0.f;
-        for (int z = 0; z < splits; ++z) {
-            const float wz = __shfl(w, z);
-            if (d < Dv)
-                a += part_acc[(((long)z * H + h) * Tn + t) * Dv + d] * wz;
+        int z = 0;
+        // four partial rows in flight per step
+        for (; z + 4 <= splits; z += 4) {
+            float x[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                x[u] = part_acc[(((long)(z + u) * H + h) * Tn + t) * Dv + dc];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) a += x[u] * __shfl(w, z + u);
         }
+        for (; z < splits; ++z)
+            a += part_acc[(((long)z * H + h) * Tn + t) * Dv + dc] *
+                 __shfl(w, z);
         if (d < Dv) stf(o + d, a * rcp);
     }
 }
@@ -1239,9 +1287,9 @@ extern "C" int launch_delta_rule(const float* q, const float* k, long qk_tok,
     if (B == 0) return 0;
     if (D > 256) return 1;
     // row groups per column: 4 unless that leaves the chip short of about
-    // two waves per SIMD (a few long portions), then 8 or 16
+    // four waves per SIMD (a few long portions), then 8 or 16
     int rg = 4;
-    while (rg < 16 && (long)B * H * ((Dv * rg + WAVE - 1) / WAVE) < 2048)
+    while (rg < 16 && (long)B * H * ((Dv * rg + WAVE - 1) / WAVE) < 4096)
         rg <<= 1;
     const int need = (D + rg - 1) / rg;
     const int dpt = need <= 4 ? 4 : need <= 8 ? 8 : need <= 16 ? 16
@@ -1274,15 +1322,16 @@ static int sink_attn_dispatch(const void* q, long q_tok, const void* k_cache,
                               float* part_acc, float* part_ml, int splits,
                               int Tn, int H, int G, int D, int Dv, int bs,
                               int window, hipStream_t s) {
-    const int dpl = (Dv + WAVE - 1) / WAVE;
+    int dpl = (Dv + WAVE - 1) / WAVE;
+    if (dpl == 3) dpl = 4;
     // query heads per wave: the largest of 4, 2, 1 that divides the group
     const int group = H / G;
     const int rep = group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
     const int units = H / rep;
-    const dim3 grid(Tn, (units + SA_WAVES - 1) / SA_WAVES, splits);
     const size_t smem = (size_t)SA_WAVES * rep * D * sizeof(float);
+    const dim3 grid(Tn, (units + SA_WAVES - 1) / SA_WAVES, splits);
     switch (dpl) {
-        SA_CASE(1) SA_CASE(2) SA_CASE(3) SA_CASE(4)
+        SA_CASE(1) SA_CASE(2) SA_CASE(4)
         default: return 1;
     }
     if (splits > 1) {
