@@ -838,11 +838,11 @@ delta_rule_kernel(const float* __restrict__ q, const float* __restrict__ k,
 // ------------------------------------------------ attention with a sink
 // Causal grouped-query softmax attention over paged keys/values
 // [n_blocks, G, bs, D|Dv], any head size up to SA_MAXD, bf16 or fp32 pages.
-// One wave per (token, query head, key split): tiles of 64 keys — for the
-// scores a lane owns ONE key and walks its row against the query held in
-// LDS (fp32), the tile's max/sum are wave reductions, and for the weighted
-// value sum lanes own output coordinates while the weights are broadcast
-// lane by lane. Scores, weights and accumulators are fp32; every score
+// One wave per (token, up to 4 query heads of one key group, key split):
+// tiles of 64 keys — for the scores a lane owns ONE key and walks its row
+// against the queries held in LDS (fp32), the tile's max/sum are wave
+// reductions, and for the weighted value sum lanes own output coordinates
+// while the weights are read lane by lane. Scores, weights and accumulators are fp32; every score
 // multiplier is already in q. The softmax denominator also counts
 // exp(sink[h]) once when sink is given. Row t at position p sees cached
 // positions j <= p (j > p - window when window > 0). With gridDim.z > 1
@@ -850,16 +850,33 @@ delta_rule_kernel(const float* __restrict__ q, const float* __restrict__ k,
 constexpr int SA_WAVES = 4;
 constexpr int SA_MAXD = 256;
 
-// scores of one key row against REP query vectors held in LDS (fp32)
-template <typename T, int REP>
-DEV_INLINE void sa_dots(const T* __restrict__ kr, const float* __restrict__ qv,
-                        int D, float* __restrict__ sc);
+// scores of one key row against REP query vectors held in LDS (fp32).
+// The row is fetched in blocks of SA_BLK 16-byte loads that are all issued
+// before any is consumed: a rolled loop of load -> use would pay one memory
+// latency per 16 bytes.
+constexpr int SA_BLK = 8;
+
 template <int REP>
 DEV_INLINE void sa_dots_f32(const float* __restrict__ kr,
                             const float* __restrict__ qv, int D,
                             float* __restrict__ sc) {
+    int d = 0;
     if (D % 4 == 0) {
-        for (int d = 0; d < D; d += 4) {
+        for (; d + 4 * SA_BLK <= D; d += 4 * SA_BLK) {
+            f32x4 x[SA_BLK];
+#pragma unroll
+            for (int c = 0; c < SA_BLK; ++c)
+                x[c] = *reinterpret_cast<const f32x4*>(kr + d + 4 * c);
+#pragma unroll
+            for (int c = 0; c < SA_BLK; ++c)
+#pragma unroll
+                for (int r = 0; r < REP; ++r) {
+                    const float* qr = qv + r * D + d + 4 * c;
+                    sc[r] += x[c][0] * qr[0] + x[c][1] * qr[1] +
+                             x[c][2] * qr[2] + x[c][3] * qr[3];
+                }
+        }
+        for (; d < D; d += 4) {
             const f32x4 x = *reinterpret_cast<const f32x4*>(kr + d);
 #pragma unroll
             for (int r = 0; r < REP; ++r) {
@@ -869,7 +886,7 @@ DEV_INLINE void sa_dots_f32(const float* __restrict__ kr,
             }
         }
     } else {
-        for (int d = 0; d < D; ++d) {
+        for (; d < D; ++d) {
             const float x = kr[d];
 #pragma unroll
             for (int r = 0; r < REP; ++r) sc[r] += x * qv[r * D + d];
@@ -880,8 +897,33 @@ template <int REP>
 DEV_INLINE void sa_dots_bf16(const unsigned short* __restrict__ kr,
                              const float* __restrict__ qv, int D,
                              float* __restrict__ sc) {
+    int d = 0;
     if (D % 8 == 0) {
-        for (int d = 0; d < D; d += 8) {
+        for (; d + 8 * SA_BLK <= D; d += 8 * SA_BLK) {
+            short8 raw[SA_BLK];
+#pragma unroll
+            for (int c = 0; c < SA_BLK; ++c)
+                raw[c] = *reinterpret_cast<const short8*>(kr + d + 8 * c);
+#pragma unroll
+            for (int c = 0; c < SA_BLK; ++c) {
+                float x[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    x[j] = bf2f((unsigned short)raw[c][j]);
+#pragma unroll
+                for (int r = 0; r < REP; ++r) {
+                    const float* qr = qv + r * D + d + 8 * c;
+                    float a = 0.f, b = 0.f;
+#pragma unroll
+                    for (int j = 0; j < 8; j += 2) {
+                        a += x[j] * qr[j];
+                        b += x[j + 1] * qr[j + 1];
+                    }
+                    sc[r] += a + b;
+                }
+            }
+        }
+        for (; d < D; d += 8) {
             float x[8];
             load_bf16x8(kr + d, x);
 #pragma unroll
@@ -897,7 +939,7 @@ DEV_INLINE void sa_dots_bf16(const unsigned short* __restrict__ kr,
             }
         }
     } else {
-        for (int d = 0; d < D; ++d) {
+        for (; d < D; ++d) {
             const float x = bf2f(kr[d]);
 #pragma unroll
             for (int r = 0; r < REP; ++r) sc[r] += x * qv[r * D + d];
@@ -941,7 +983,10 @@ sink_attn_kernel(const T* __restrict__ q, long q_tok,
     const int p = positions[t];
     const int g = h0 / (H / G);
     const int lo = window > 0 ? max(0, p - window + 1) : 0;
-    const int per = (p + 1 - lo + nsplit - 1) / nsplit;
+    // a split takes whole 64-key tiles, so no wave pays a full score pass
+    // for a few keys; splits past the end stay empty (sum 0) for the merge
+    const int per =
+        ((p + 1 - lo + nsplit - 1) / nsplit + WAVE - 1) / WAVE * WAVE;
     const int klo = lo + split * per, khi = min(p + 1, klo + per);
     float* qv = sa_q + (long)wid * REP * D;
     for (int i = lane; i < REP * D; i += WAVE)
