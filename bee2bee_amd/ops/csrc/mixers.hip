@@ -962,7 +962,24 @@ template <int REP> struct SaDots<unsigned short, REP> {
 // the group size), so each cached row is read once for all of them.
 constexpr int SA_PV = 8;      // value rows in flight per step
 
-template <typename T, int DPL, int REP>
+// Output coordinate i of a lane. PAIR (even value size): a lane owns
+// neighbouring coordinates 2*lane, 2*lane+1 (+128 per further pair) and
+// fetches both with one load; otherwise lane, lane+64, ...
+template <bool PAIR> DEV_INLINE int sa_coord(int lane, int i) {
+    return PAIR ? (i >> 1) * (2 * WAVE) + 2 * lane + (i & 1) : lane + i * WAVE;
+}
+DEV_INLINE void sa_ld2(const float* p, float& a, float& b) {
+    const float2v w = *reinterpret_cast<const float2v*>(p);
+    a = w[0];
+    b = w[1];
+}
+DEV_INLINE void sa_ld2(const unsigned short* p, float& a, float& b) {
+    const unsigned int w = *reinterpret_cast<const unsigned int*>(p);
+    a = bf2f((unsigned short)(w & 0xffffu));
+    b = bf2f((unsigned short)(w >> 16));
+}
+
+template <typename T, int DPL, int REP, bool PAIR>
 __global__ void __launch_bounds__(SA_WAVES * WAVE)
 sink_attn_kernel(const T* __restrict__ q, long q_tok,
                  const T* __restrict__ k_cache, const T* __restrict__ v_cache,
@@ -1029,10 +1046,19 @@ sink_attn_kernel(const T* __restrict__ q, long q_tok,
             for (int u = 0; u < SA_PV; ++u) {
                 const T* vr =
                     v_cache + (long)__builtin_amdgcn_readlane(row, jj + u) * Dv;
+                if constexpr (PAIR) {
 #pragma unroll
-                for (int i = 0; i < DPL; ++i) {
-                    const int d = lane + i * WAVE;
-                    vv[u][i] = d < Dv ? ldf(vr + d) : 0.f;
+                    for (int i = 0; i < DPL; i += 2) {
+                        const int d = sa_coord<true>(lane, i);
+                        vv[u][i] = vv[u][i + 1] = 0.f;
+                        if (d < Dv) sa_ld2(vr + d, vv[u][i], vv[u][i + 1]);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < DPL; ++i) {
+                        const int d = sa_coord<false>(lane, i);
+                        vv[u][i] = d < Dv ? ldf(vr + d) : 0.f;
+                    }
                 }
             }
 #pragma unroll
@@ -1063,7 +1089,7 @@ sink_attn_kernel(const T* __restrict__ q, long q_tok,
             T* o = out + (long)t * out_tok + (long)h * Dv;
 #pragma unroll
             for (int i = 0; i < DPL; ++i) {
-                const int d = lane + i * WAVE;
+                const int d = sa_coord<PAIR>(lane, i);
                 if (d < Dv) stf(o + d, acc[r][i] * rcp);
             }
         } else {
@@ -1074,7 +1100,7 @@ sink_attn_kernel(const T* __restrict__ q, long q_tok,
             }
 #pragma unroll
             for (int i = 0; i < DPL; ++i) {
-                const int d = lane + i * WAVE;
+                const int d = sa_coord<PAIR>(lane, i);
                 if (d < Dv) part_acc[prow * Dv + d] = acc[r][i];
             }
         }
@@ -1345,18 +1371,19 @@ extern "C" int launch_delta_rule(const float* q, const float* k, long qk_tok,
     return 1;
 }
 
-#define SA_LAUNCH(N, R)                                                       \
-    sink_attn_kernel<TT, N, R><<<grid, SA_WAVES * WAVE, smem, s>>>(           \
+#define SA_LAUNCH(N, R, P)                                                    \
+    sink_attn_kernel<TT, N, R, P><<<grid, SA_WAVES * WAVE, smem, s>>>(        \
         (const TT*)q, q_tok, (const TT*)k_cache, (const TT*)v_cache,          \
         block_table, bt_stride, positions, seq_idx, sink, (TT*)out, out_tok,  \
         out_scale, part_acc, part_ml, Tn, H, G, D, Dv, bs, window)
 
-#define SA_CASE(N)                                                            \
-    case N:                                                                   \
-        if (rep == 4) SA_LAUNCH(N, 4);                                        \
-        else if (rep == 2) SA_LAUNCH(N, 2);                                   \
-        else SA_LAUNCH(N, 1);                                                 \
-        break;
+#define SA_CASE(N, P)                                                         \
+    if (dpl == N && pair == P) {                                              \
+        if (rep == 4) SA_LAUNCH(N, 4, P);                                     \
+        else if (rep == 2) SA_LAUNCH(N, 2, P);                                \
+        else SA_LAUNCH(N, 1, P);                                              \
+        launched = true;                                                      \
+    }
 
 template <typename TT>
 static int sink_attn_dispatch(const void* q, long q_tok, const void* k_cache,
@@ -1367,7 +1394,10 @@ static int sink_attn_dispatch(const void* q, long q_tok, const void* k_cache,
                               float* part_acc, float* part_ml, int splits,
                               int Tn, int H, int G, int D, int Dv, int bs,
                               int window, hipStream_t s) {
-    int dpl = (Dv + WAVE - 1) / WAVE;
+    // even value sizes: a lane owns coordinate pairs (one load for two)
+    const bool pair = Dv % 2 == 0;
+    int dpl = pair ? 2 * ((Dv + 2 * WAVE - 1) / (2 * WAVE))
+                   : (Dv + WAVE - 1) / WAVE;
     if (dpl == 3) dpl = 4;
     // query heads per wave: the largest of 4, 2, 1 that divides the group
     const int group = H / G;
@@ -1375,10 +1405,10 @@ static int sink_attn_dispatch(const void* q, long q_tok, const void* k_cache,
     const int units = H / rep;
     const size_t smem = (size_t)SA_WAVES * rep * D * sizeof(float);
     const dim3 grid(Tn, (units + SA_WAVES - 1) / SA_WAVES, splits);
-    switch (dpl) {
-        SA_CASE(1) SA_CASE(2) SA_CASE(4)
-        default: return 1;
-    }
+    bool launched = false;
+    SA_CASE(2, true) SA_CASE(4, true)
+    SA_CASE(1, false) SA_CASE(2, false) SA_CASE(4, false)
+    if (!launched) return 1;
     if (splits > 1) {
         const dim3 g2(Tn, (H + SA_WAVES - 1) / SA_WAVES);
         sink_attn_combine_kernel<TT><<<g2, SA_WAVES * WAVE, 0, s>>>(

@@ -150,7 +150,7 @@ def test_head_gated_norm(dtype, H, Dv, weighted, act):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,D,dims,window", [
     (6, 3, 64, 16, 0), (4, 1, 40, 40, 0), (2, 2, 24, 0, 0), (8, 2, 128, 64, 0),
-    (4, 2, 72, 8, 5), (3, 3, 200, 100, 0), (2, 1, 20, 4, 0), (6, 1, 12, 12, 3)])
+    (4, 2, 72, 8, 5), (3, 3, 200, 100, 0), (2, 1, 20, 4, 0), (6, 1, 12, 12, 3), (2, 1, 21, 0, 0), (4, 4, 160, 32, 0)])
 def test_sink_attention(dtype, H, G, D, dims, window):
     torch.manual_seed(6)
     bs, nb = 16, 24
