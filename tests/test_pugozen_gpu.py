@@ -126,3 +126,26 @@ def test_graph_decode_equals_eager(tmp_path):
         if float(top2[0] - top2[1]) > 1e-3:
             assert int(logits.argmax()) == tok
         seq.append(tok)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_head_size_of_the_matrix_core_path(tmp_path, dtype):
+    """Attention heads of 64: bf16 prompt portions of 16 tokens or more run
+    on the matrix cores (paged prompt kernel, weights as a bf16 pair, sink in
+    its epilogue), shorter portions and decode rows on the generic kernel
+    with its key split; fp32 takes the generic kernel throughout. All of
+    them must agree with the oracle on one sequence cut in different ways."""
+    cfg = O.make_config(order=("parallel", "delta", "parallel"),
+                        shared=((2, 0),), width=64, vocab=90, ff=72, heads=4,
+                        kv_heads=2, dim=64, rot_dims=32, scale=0.125,
+                        r_heads=2, r_kv_heads=2, r_dim=16, r_vdim=16)
+    W = O.random_weights(cfg, seed=25)
+    eng = make_engine(tmp_path, cfg, W, device="cuda", dtype=dtype,
+                      kv_blocks=40)
+    toks = random_tokens(210, cfg["vocab"], 11)
+    want = oracle_logits(cfg, W, toks)
+    for sched in ([[("a", 210)]],
+                  chunk_schedule("a", 210, [100, 3, 60, 17, 1, 16]),
+                  [[("a", 170)]] + [[("a", 1)]] * 40):
+        got = replay(eng, {"a": toks}, sched)["a"]
+        assert_logits(got, want, dtype)
